@@ -1,0 +1,172 @@
+#!/usr/bin/env python3
+"""Benchmark of the differentiable Gaussian ray-march path on one MI355X.
+
+One step = one training view through the reference's operator API:
+``RenderOptixFunction.apply`` (k-sigma boxes + LBVH build + SH colour + prim packing +
+forward march) followed by the backward of an MSE loss (backward march + SH backward),
+exactly what scripts/train.py:119-148 runs per iteration (the reference rebuilds its
+acceleration structure on every forward, ``update=False``).
+
+Workload (``config.workload``): the 1 M-Gaussian scene of the training-stress configuration
+(centres uniform in a ball of radius 2) rendered at 800x800 -- the configuration the headline
+metric "Mrays/s fwd+bwd @1M Gaussians 800x800" is quoted on -- one camera of the
+upper-hemisphere orbit per step.  Inputs are resident in HBM before the timed region.
+
+Prints ONE JSON line.  ``roofline`` prices the dominant kernel (the backward march) with its
+algorithmic bytes (64+56 B per ray-slab-hit + 24 B per ray) over its own HIP-event time;
+``cpu_baseline`` times the CPU oracle on a bounded ray sample of the same workload.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+from raygaussx_amd import _lib as L  # noqa: E402
+from raygaussx_amd import optix_utils as u_ox  # noqa: E402
+from raygaussx_amd import scenes  # noqa: E402
+from raygaussx_amd.render_optix import RenderOptixFunction, default_settings  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per k_march_bwd launch of the default workload, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE runs scaled by a copy kernel of known size (profiles/); None until measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+WORKLOADS = {
+    # name: (scene config, n, width, height)
+    "c4_1M_800x800": (4, 1_000_000, 800, 800),
+    "c1_300k_800x800": (1, 300_000, 800, 800),
+    "c4_1M_1024x1024": (4, 1_000_000, 1024, 1024),
+    "c0_4096_128x128": (0, 4096, 128, 128),
+}
+
+
+def cpu_baseline(scene, cam, cfg, n_sample, threads):
+    """Forward + backward of the CPU oracle on a strided ray sample of the same view."""
+    from oracle import oracle as orc
+    orc.build()
+    orc.set_num_threads(threads)
+    sc = scenes.scene_to_numpy(scene)
+    n_rays = cam.image_width * cam.image_height
+    ids = np.linspace(0, n_rays - 1, n_sample).astype(np.int64)
+    t0 = time.perf_counter()
+    img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
+                                      ray_ids=ids)
+    dloss = np.full(img.shape, 1.0 / img.size, np.float32)
+    orc.render_backward(sc, ctx, img, dloss)
+    dt = time.perf_counter() - t0
+    return dict(value=round(n_sample / dt / 1e6, 6), unit="Mrays/s", cores=threads, kind="port",
+                sample=f"{n_sample} strided rays of camera 0, fwd+bwd, all {sc['positions'].shape[0]} Gaussians "
+                       f"(brute-force hit search), {dt:.1f} s")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c4_1M_800x800", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-rays", type=int, default=1024, help="ray sample of the CPU baseline (0 = skip)")
+    ap.add_argument("--forward-only", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (--gpus 1); the path shards by views/tiles, "
+                 "see DESIGN.md, but no multi-GPU figure is produced")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: needs a GPU (librgx has no CPU path)")
+    dev = "cuda:0"
+    L.lib()
+    config, n, width, height = WORKLOADS[args.workload]
+    cfg = dict(scenes.CONFIGS[config])
+    scene = scenes.make_scene(config, n=n)
+    dscene = {k: v.to(dev) for k, v in scene.items()}
+    names = ("positions", "scales", "quaternions", "densities", "color_features", "sph_gauss_features",
+             "bandwidth_sharpness", "lobe_axis")
+    params = [dscene[k].clone().requires_grad_(not args.forward_only) for k in names]
+    n_cams = min(cfg["n_cameras"], 100)
+    cams = [scenes.make_camera(config, i, width=width, height=height).to(dev) for i in range(n_cams)]
+    n_rays = width * height
+    target = torch.rand(n_rays, 3, device=dev, generator=torch.Generator(dev).manual_seed(1))
+    stats = u_ox.new_stats(dev)
+    gas = None
+
+    def step(i):
+        nonlocal gas
+        s = default_settings(cams[i % n_cams], cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
+                             t_eps=cfg["t_eps"], gas=gas)
+        s.stats = stats
+        img = RenderOptixFunction.apply(*params, s)
+        gas = s.gas
+        if not args.forward_only:
+            loss = ((img - target) ** 2).mean()
+            loss.backward()
+            for p in params:
+                p.grad = None
+        return img
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    stats.zero_()
+    L.timing_enable(True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(args.warmup + i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    timing = L.timing_read()
+    L.timing_enable(False)
+    st = u_ox.read_stats(stats)
+
+    ms_per_step = elapsed / args.steps * 1e3
+    mrays = n_rays * args.steps / elapsed / 1e6
+    passes = 1 if args.forward_only else 2
+    hits_per_launch = st["hit_pairs"] / (args.steps * passes)   # H: fwd and bwd march the same slabs
+    if args.forward_only:
+        kname, alg_bytes = "march_forward", 64.0 * hits_per_launch + 12.0 * n_rays
+    else:
+        kname, alg_bytes = "march_backward", (64.0 + 56.0) * hits_per_launch + 24.0 * n_rays
+    k_ms, k_cnt = timing[kname]
+    k_avg_ms = k_ms / max(k_cnt, 1)
+    achieved = alg_bytes / (k_avg_ms * 1e-3) / 1e9 if k_avg_ms > 0 else 0.0
+    roofline = dict(bound="hbm", kernel="k_" + kname.replace("march_forward", "march_fwd").replace("march_backward", "march_bwd"),
+                    achieved=round(achieved, 2), peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 5),
+                    traffic=MEASURED_TRAFFIC_BYTES.get((args.workload, kname)),
+                    kernel_ms=round(k_avg_ms, 4), algorithmic_bytes=int(alg_bytes),
+                    hit_pairs_per_launch=int(hits_per_launch))
+    # whole-step roofline-derived rate: all algorithmic bytes of one step at peak bandwidth
+    step_bytes = (64.0 * hits_per_launch + 12.0 * n_rays + 300.0 * n
+                  + (0 if args.forward_only else (120.0 * hits_per_launch + 24.0 * n_rays + 464.0 * n)))
+    out = dict(metric="Mrays/s fwd" + ("" if args.forward_only else "+bwd"), value=round(mrays, 4), unit="Mrays/s",
+               n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_per_step, 4),
+               higher_is_better=True, scaling="weak", vs_baseline=None, dtype="f32", data="synthetic",
+               config=dict(workload=args.workload, gaussians=n, width=width, height=height, sh_degree=3,
+                           dt_step=cfg["dt_step"], dynamic_sampling=cfg["dynamic_sampling"],
+                           max_prim_slice=cfg["max_prim_slice"], step="bvh build + sh + pack + march fwd"
+                           + ("" if args.forward_only else " + march bwd + sh bwd") + ", 1 view"),
+               roofline=roofline,
+               step_roofline=dict(bytes_per_step=int(step_bytes),
+                                  achieved=round(step_bytes / (ms_per_step * 1e-3) / 1e9, 2), unit="GB/s",
+                                  frac=round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
+                                  roofline_mrays=round(HBM_PEAK_GBPS * 1e9 * n_rays / step_bytes / 1e6, 2)),
+               kernels_ms={k: round(v[0] / max(v[1], 1), 4) for k, v in timing.items() if v[1]},
+               stats_per_step={k: v / args.steps for k, v in st.items()})
+    if args.cpu_rays > 0:
+        threads = min(16, os.cpu_count() or 1)
+        out["cpu_baseline"] = cpu_baseline(scene, scenes.make_camera(config, 0, width=width, height=height), cfg,
+                                           args.cpu_rays, threads)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,193 @@
+/*
+ * rgx.h -- C ABI of librgx.so: the MI355X (gfx950) implementation of the
+ * RayGaussX differentiable Gaussian ray-marching renderer.
+ *
+ * Every entry point replaces a piece of the reference's OptiX/CuPy host glue
+ * (paths relative to the reference tree).  Conventions:
+ *   - all pointers are DEVICE pointers on the current HIP device unless the
+ *     parameter is documented as "host";
+ *   - `stream` is a hipStream_t passed as void* (0 = the null stream); every
+ *     call only enqueues work on it and never synchronises, except the two
+ *     explicitly synchronous read-back helpers;
+ *   - the caller owns every buffer, including the workspaces whose sizes the
+ *     *_bytes queries return; the library never allocates device memory;
+ *   - return 0 on success or a negative RGX_E* code; nothing throws or exits.
+ *     rgx_strerror() names a code, rgx_last_hip_error() returns the hipError_t
+ *     behind the calling thread's last RGX_EHIP.
+ * Calls are thread-compatible (the autograd engine calls the backward from
+ * its own thread); two calls that share a workspace must be ordered by the
+ * stream.
+ */
+#ifndef RGX_H
+#define RGX_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RGX_ABI_VERSION 1
+
+#define RGX_OK 0
+#define RGX_EINVAL -1     /* bad argument (null pointer, negative size, unsupported degree ...) */
+#define RGX_EWORKSPACE -2 /* workspace too small or misaligned */
+#define RGX_EHIP -3       /* a HIP runtime call failed; see rgx_last_hip_error() */
+
+/* Launch constants of one view.  Mirrors the camera part of `Params`
+ * (optix_raycasting/cuda_train/forward/gaussians_aabb.h:14-44) as filled at
+ * optix_raycasting/optix_utils.py:252-266.  Host struct. */
+typedef struct RgxCamera {
+    float eye[3];       /* camera.camera_center */
+    float u[3];         /* world_view_transform[:3,0]  (camera right, world space) */
+    float v[3];         /* world_view_transform[:3,1]  (camera down) */
+    float w[3];         /* world_view_transform[:3,2]  (camera forward) */
+    float tan_half_fov_x, tan_half_fov_y, principal_x, principal_y; /* cam_intr */
+    int32_t width, height; /* already multiplied by the supersampling factors */
+} RgxCamera;
+
+/* Marching constants.  dt_step / dynamic_sampling / max_prim_slice /
+ * white_background are `Params` fields; t_eps is TRANSMITTANCE_EPSILON
+ * (gaussians_aabb.h:4, 0.001f in the reference) made a run-time value. Host struct. */
+typedef struct RgxMarch {
+    float dt_step;
+    int32_t dynamic_sampling;
+    int32_t max_prim_slice;
+    int32_t white_background;
+    float t_eps;
+} RgxMarch;
+
+/* Optional device-side counters, accumulated (not reset) by the march kernels. */
+typedef struct RgxStats {
+    unsigned long long hit_pairs;     /* sum over blended slabs of the hit-list length */
+    unsigned long long slabs;         /* slabs blended */
+    unsigned long long empty_slabs;   /* collect queries that found nothing */
+    unsigned long long overflow_rays; /* collect queries truncated at max_prim_slice */
+    unsigned long long rays_hit;      /* rays whose first-hit query found a Gaussian */
+    unsigned long long nodes_visited; /* BVH nodes fetched by all queries */
+} RgxStats;
+
+int rgx_abi_version(void);
+const char *rgx_strerror(int code);
+int rgx_last_hip_error(void);
+
+/* ---- per-Gaussian kernels ------------------------------------------------ */
+
+/* Replaces ellipsoids_bbox_from_quat (optix_utils.py:36-109): k-sigma AABB of
+ * every Gaussian plus the scene bounding box.  bboxes (N,6) = xmin,ymin,zmin,
+ * xmax,ymax,zmax; bb_min/bb_max (3) device floats.  Any output may be NULL. */
+int rgx_aabb(const float *pos, const float *scale, const float *quat, const float *dens, int64_t n,
+             float sigma_threshold, float *bboxes, float *bb_min, float *bb_max, void *stream);
+
+/* Replaces forward_sh (utils/sh_utils.cu:122-216) as launched by compute_cupy_rgb
+ * (render_optix.py:19-32).  sh is (N,3,K) channel-major, K=(degree+1)^2, degree 0..3;
+ * sg (N,3,G), sharp (N,G), axis (N,G,3) may be NULL when G == 0.  eye: host float[3]. */
+int rgx_sh_forward(const float *eye, const float *pos, const float *sh, const float *sg,
+                   const float *sharp, const float *axis, int32_t g, int32_t degree, int64_t n,
+                   float *rgb, void *stream);
+
+/* Replaces backward_sh (utils/sh_utils.cu:218-412) as launched by compute_cupy_sh_grad
+ * (render_optix.py:34-52).  Writes (does not accumulate) dsh (N,3,K), dpos (N,3) and,
+ * when G > 0, dsg / dsharp / daxis.  Keeps the reference's d/dy term of basis 9
+ * (sh_utils.cu:367).  eye: host float[3]. */
+int rgx_sh_backward(const float *eye, const float *pos, const float *sh, const float *sg,
+                    const float *sharp, const float *axis, int32_t g, int32_t degree, int64_t n,
+                    const float *drgb, float *dsh, float *dpos, float *dsg, float *dsharp,
+                    float *daxis, void *stream);
+
+/* ---- acceleration structure ---------------------------------------------- */
+
+/* Replaces create_acceleration_structure (optix_utils.py:139-142; the OptiX
+ * GAS build) together with the AABB pass that feeds it: k-sigma AABBs, scene
+ * bbox, 63-bit Morton codes of the centres, radix sort, Karras radix tree,
+ * bottom-up refit, skip links.  The result lives in `ws` (device memory of at
+ * least rgx_build_workspace_bytes(n) bytes, 256-byte aligned) and stays valid
+ * until the next build into the same buffer; reuse it across views. */
+int rgx_build_workspace_bytes(int64_t n, size_t *bytes);
+int rgx_build(const float *pos, const float *scale, const float *quat, const float *dens, int64_t n,
+              float sigma_threshold, void *ws, size_t ws_bytes, void *stream);
+
+/* Same tree over caller-supplied boxes (N,6), the literal signature of
+ * create_acceleration_structure(ctx, bboxes) (optix_utils.py:139-142). */
+int rgx_build_aabbs(const float *bboxes, int64_t n, void *ws, size_t ws_bytes, void *stream);
+
+/* Synchronous read-back of the scene bbox held in a built workspace
+ * (host out[6] = min xyz, max xyz); what bb_min.get()/bb_max.get() returned at
+ * optix_utils.py:254-255.  Waits for `stream`. */
+int rgx_scene_bbox(const void *ws, float *host_out6, void *stream);
+/* The build's permutation: order[j] = input index of the j-th Gaussian in Morton order. */
+int rgx_build_order(const void *ws, int64_t n, int32_t *order_out, void *stream);
+
+/* Replaces the prim packing at optix_utils.py:268-304: the 64-byte PrimData record
+ * (gaussians_aabb.h:7-12) of every Gaussian, written in the build's Morton order
+ * when `ws` is a built workspace, or in input order when ws == NULL.
+ * eye: host float[3].  prims: (N,16) floats, 64-byte aligned. */
+int rgx_pack_prims(const void *ws, const float *eye, const float *pos, const float *scale,
+                   const float *quat, const float *dens, const float *rgb, int64_t n,
+                   float sigma_threshold, float *prims, void *stream);
+
+/* ---- ray march ------------------------------------------------------------ */
+
+/* Scratch for one march launch: the backward's Morton-ordered gradient block
+ * and the overflow part of the per-ray hit lists (the reference's hit_prim_idx,
+ * optix_utils.py:306). */
+int rgx_march_workspace_bytes(int64_t n, int64_t n_rays, int32_t max_prim_slice, size_t *bytes);
+
+/* Replaces launch_pipeline_forward / launch_pipeline_test (optix_utils.py:222-322,
+ * 503-601) and the OptiX programs of cuda_train/forward/gaussians_aabb.cu:
+ * ray_colors (W*H,3), row-major pixels.  cam, march: host structs.
+ * prims: from rgx_pack_prims with the same ws.  stats may be NULL. */
+int rgx_march_forward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims,
+                      int64_t n, float *ray_colors, void *march_ws, size_t march_ws_bytes,
+                      RgxStats *stats, void *stream);
+
+/* Replaces launch_pipeline_backward + reduce_temp_grads (optix_utils.py:325-500) and
+ * cuda_train/backward/gaussians_aabb.cu: gradients of sum(dloss * ray_colors) with
+ * respect to density (N), rgb (N,3), position (N,3), scale (N,3), quaternion (N,4),
+ * in INPUT order, overwritten.  ray_colors is the forward's output. */
+int rgx_march_backward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims,
+                       int64_t n, const float *ray_colors, const float *dloss, float *ddens,
+                       float *drgb, float *dpos, float *dscale, float *dquat, void *march_ws,
+                       size_t march_ws_bytes, RgxStats *stats, void *stream);
+
+/* Test hooks: the two OptiX ray queries on caller-supplied segments (origin = eye,
+ * host float[3]; dirs (n,3); tlo/thi (n)).  first-hit: optixTrace SBT offset 0
+ * (gaussians_aabb.cu:234-247, 370-380), out_t = smallest hit t or -1.  collect:
+ * optixTrace SBT offset 1 + __anyhit__ah (gaussians_aabb.cu:282-295, 349-367),
+ * counts[i] = number of hits (negated when truncated at cap), ids (n,cap) = INPUT
+ * indices in traversal order. */
+int rgx_first_hit(const void *ws, const float *prims, int64_t n_prims, const float *eye, int64_t n,
+                  const float *dirs, const float *tlo, const float *thi, float *out_t, void *stream);
+int rgx_trace_segments(const void *ws, const float *prims, int64_t n_prims, const float *eye, int64_t n,
+                       const float *dirs, const float *tlo, const float *thi, int32_t cap,
+                       int32_t *counts, int32_t *ids, void *stream);
+
+/* ---- Morton reordering of the point cloud --------------------------------- */
+
+/* Replaces quantify_pos_min_max + morton_code + argsort (utils/reordering_utils.py:55-104,
+ * classes/point_cloud.py:1017-1024): 10 bits per axis on the positions' own min/max,
+ * x -> bit 3i, y -> 3i+1, z -> 3i+2; order = stable ascending sort of the codes.
+ * codes (N) int64 and order (N) int64 outputs; either may be NULL. */
+int rgx_morton_workspace_bytes(int64_t n, size_t *bytes);
+int rgx_morton_order(const float *pos, int64_t n, int64_t *codes, int64_t *order, void *ws,
+                     size_t ws_bytes, void *stream);
+
+/* ---- measurement ----------------------------------------------------------- */
+
+/* Per-kernel timing with HIP events recorded on the launch stream around the kernels
+ * of each entry point (what the reference's commented-out CUDA-event code at
+ * optix_utils.py:466-485 and scripts/test.py:109-126 measured).  Off by default.
+ * ids: 0 build, 1 sh_forward, 2 pack_prims, 3 march_forward (the k_march_fwd launch
+ * only), 4 march_backward (the k_march_bwd launch only), 5 unpermute_grads,
+ * 6 sh_backward.  rgx_timing_read waits for the recorded events and returns the
+ * summed milliseconds and the number of launches since the last reset. */
+int rgx_timing_enable(int on);
+int rgx_timing_reset(void);
+const char *rgx_timing_name(int id);
+int rgx_timing_read(int id, double *total_ms, int64_t *launches);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RGX_H */

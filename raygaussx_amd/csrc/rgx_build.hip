@@ -1,0 +1,590 @@
+// LBVH construction on the GPU: k-sigma AABBs + scene bbox, 63-bit Morton
+// codes, LDS-staged LSD radix sort, Karras radix tree, bottom-up refit, skip
+// links.  Replaces the OptiX GAS build (optix_raycasting/optix_utils.py:139-142)
+// and the AABB pass feeding it (optix_utils.py:36-109).  Also hosts the 30-bit
+// Morton ordering of the point cloud (utils/reordering_utils.py:55-104).
+#include "rgx_device.h"
+
+// ---------------------------------------------------------------------------
+// order-preserving float <-> int encoding for atomicMin/atomicMax
+__device__ __forceinline__ int32_t enc_f(float f)
+{
+    int32_t i = __float_as_int(f);
+    return i >= 0 ? i : i ^ 0x7fffffff;
+}
+__device__ __forceinline__ float dec_f(int32_t i) { return __int_as_float(i >= 0 ? i : i ^ 0x7fffffff); }
+
+__global__ void k_init_header(WsHeader *h, int64_t n)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        for (int a = 0; a < 3; ++a) {
+            h->bb_min_enc[a] = enc_f(INFINITY);
+            h->bb_max_enc[a] = enc_f(-INFINITY);
+            h->bb_min[a] = INFINITY;
+            h->bb_max[a] = -INFINITY;
+        }
+        h->n = n;
+        h->root = 0;
+        h->built = 0;
+    }
+}
+
+__device__ __forceinline__ float wave_min(float v)
+{
+    for (int o = 32; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v)
+{
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+
+// k-sigma AABB of a rotated ellipsoid (optix_utils.py:49-77), canonical arithmetic.
+__global__ __launch_bounds__(256) void k_aabb(const float *__restrict__ pos, const float *__restrict__ scale,
+                                              const float *__restrict__ quat, const float *__restrict__ dens,
+                                              int64_t n, float thr, float *__restrict__ boxes, int32_t *mn_enc, int32_t *mx_enc)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    float b[6] = {INFINITY, INFINITY, INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    if (i < n) {
+        const float t = dens[i] / thr;
+        float d = canon_logf(t * t);
+        if (!(d > 0.0f)) d = 0.0f;
+        d = sqrtf(d);
+        float W = quat[4 * i], X = quat[4 * i + 1], Y = quat[4 * i + 2], Z = quat[4 * i + 3];
+        const float nn = ((W * W + X * X) + Y * Y) + Z * Z;
+        const float invn = 1.0f / sqrtf(nn + 1e-20f);
+        W *= invn; X *= invn; Y *= invn; Z *= invn;
+        const float L1x = 1.f - 2.f * (Y * Y + Z * Z), L1y = 2.f * (X * Y - W * Z), L1z = 2.f * (X * Z + W * Y);
+        const float L2x = 2.f * (X * Y + W * Z), L2y = 1.f - 2.f * (X * X + Z * Z), L2z = 2.f * (Y * Z - W * X);
+        const float L3x = 2.f * (X * Z - W * Y), L3y = 2.f * (Y * Z + W * X), L3z = 1.f - 2.f * (X * X + Y * Y);
+        const float s0 = scale[3 * i], s1 = scale[3 * i + 1], s2 = scale[3 * i + 2];
+        const float hx = d * sqrtf(((s0 * L1x) * (s0 * L1x) + (s1 * L1y) * (s1 * L1y)) + (s2 * L1z) * (s2 * L1z));
+        const float hy = d * sqrtf(((s0 * L2x) * (s0 * L2x) + (s1 * L2y) * (s1 * L2y)) + (s2 * L2z) * (s2 * L2z));
+        const float hz = d * sqrtf(((s0 * L3x) * (s0 * L3x) + (s1 * L3y) * (s1 * L3y)) + (s2 * L3z) * (s2 * L3z));
+        const float c0 = pos[3 * i], c1 = pos[3 * i + 1], c2 = pos[3 * i + 2];
+        b[0] = c0 - hx; b[1] = c1 - hy; b[2] = c2 - hz;
+        b[3] = c0 + hx; b[4] = c1 + hy; b[5] = c2 + hz;
+        if (boxes)
+            for (int a = 0; a < 6; ++a) boxes[6 * i + a] = b[a];
+    }
+    __shared__ float red[4][6];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int a = 0; a < 3; ++a) {
+        const float mn = wave_min(b[a]), mx = wave_max(b[a + 3]);
+        if (lane == 0) { red[wave][a] = mn; red[wave][a + 3] = mx; }
+    }
+    __syncthreads();
+    if (threadIdx.x < 3 && mn_enc) {
+        const int a = threadIdx.x;
+        const float mn = fminf(fminf(red[0][a], red[1][a]), fminf(red[2][a], red[3][a]));
+        const float mx = fmaxf(fmaxf(red[0][a + 3], red[1][a + 3]), fmaxf(red[2][a + 3], red[3][a + 3]));
+        atomicMin(&mn_enc[a], enc_f(mn));
+        atomicMax(&mx_enc[a], enc_f(mx));
+    }
+}
+
+// stand-alone reductions keep their encoded running min/max in the output buffers themselves
+__global__ void k_init_enc(int32_t *mn, int32_t *mx)
+{
+    if (threadIdx.x < 3) {
+        mn[threadIdx.x] = enc_f(INFINITY);
+        mx[threadIdx.x] = enc_f(-INFINITY);
+    }
+}
+__global__ void k_decode_enc(int32_t *mn, int32_t *mx)
+{
+    if (threadIdx.x < 3) {
+        ((float *)mn)[threadIdx.x] = dec_f(mn[threadIdx.x]);
+        ((float *)mx)[threadIdx.x] = dec_f(mx[threadIdx.x]);
+    }
+}
+
+__global__ void k_finish_bbox(WsHeader *h, float *bb_min, float *bb_max)
+{
+    const int a = threadIdx.x;
+    if (a < 3) {
+        const float mn = dec_f(h->bb_min_enc[a]), mx = dec_f(h->bb_max_enc[a]);
+        h->bb_min[a] = mn;
+        h->bb_max[a] = mx;
+        if (bb_min) bb_min[a] = mn;
+        if (bb_max) bb_max[a] = mx;
+    }
+}
+
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ uint64_t expand21(uint64_t x)
+{
+    x &= 0x1fffffull;
+    x = (x | x << 32) & 0x1f00000000ffffull;
+    x = (x | x << 16) & 0x1f0000ff0000ffull;
+    x = (x | x << 8) & 0x100f00f00f00f00full;
+    x = (x | x << 4) & 0x10c30c30c30c30c3ull;
+    x = (x | x << 2) & 0x1249249249249249ull;
+    return x;
+}
+
+// 21 bits per axis of the box centre, relative to the scene bbox
+__global__ __launch_bounds__(256) void k_morton63(const float *__restrict__ boxes, int64_t n, const WsHeader *hdr,
+                                                  uint64_t *__restrict__ keys, uint32_t *__restrict__ vals)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint64_t q[3];
+    for (int a = 0; a < 3; ++a) {
+        const float lo = hdr->bb_min[a], ext = hdr->bb_max[a] - lo;
+        const float c = 0.5f * boxes[6 * i + a] + 0.5f * boxes[6 * i + 3 + a];
+        float u = ext > 0.f ? (c - lo) / ext : 0.f;
+        u = fminf(fmaxf(u, 0.f), 1.f);
+        const float s = u * 2097152.0f;
+        q[a] = s >= 2097151.0f ? 2097151ull : (uint64_t)s;
+    }
+    keys[i] = (expand21(q[0]) << 2) | (expand21(q[1]) << 1) | expand21(q[2]);
+    vals[i] = (uint32_t)i;
+}
+
+// ---------------------------------------------------------------------------
+// LSD radix sort, 8 bits per pass, keys u64 + values u32, stable.  Per pass:
+// per-tile digit histogram -> exclusive scan over (digit, tile) -> scatter.
+// The scatter keeps its per-wave digit cursors in LDS and ranks the 64 keys a
+// wave handles at a time with ballot matching, so equal digits leave in input
+// order.
+template <typename K>
+__global__ __launch_bounds__(RGX_RS_THREADS) void k_rs_hist(const K *__restrict__ keys, int64_t n, int shift,
+                                                            uint32_t *__restrict__ hist, int nblocks)
+{
+    __shared__ uint32_t h[256];
+    h[threadIdx.x] = 0;
+    __syncthreads();
+    const int64_t base = (int64_t)blockIdx.x * RGX_RS_TILE;
+    for (int r = 0; r < RGX_RS_ITEMS; ++r) {
+        const int64_t i = base + r * RGX_RS_THREADS + threadIdx.x;
+        if (i < n) atomicAdd(&h[(uint32_t)(keys[i] >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    hist[(size_t)threadIdx.x * nblocks + blockIdx.x] = h[threadIdx.x];
+}
+
+__global__ __launch_bounds__(1024) void k_rs_scan(uint32_t *__restrict__ hist, int64_t total)
+{
+    __shared__ uint32_t part[1024];
+    const int64_t per = (total + 1023) / 1024;
+    const int64_t b = threadIdx.x * per, e = b + per < total ? b + per : total;
+    uint32_t s = 0;
+    for (int64_t i = b; i < e; ++i) s += hist[i];
+    part[threadIdx.x] = s;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) { // Hillis-Steele inclusive scan
+        uint32_t v = threadIdx.x >= o ? part[threadIdx.x - o] : 0;
+        __syncthreads();
+        part[threadIdx.x] += v;
+        __syncthreads();
+    }
+    uint32_t run = threadIdx.x ? part[threadIdx.x - 1] : 0;
+    for (int64_t i = b; i < e; ++i) {
+        const uint32_t v = hist[i];
+        hist[i] = run;
+        run += v;
+    }
+}
+
+template <typename K>
+__global__ __launch_bounds__(RGX_RS_THREADS) void k_rs_scatter(const K *__restrict__ kin, const uint32_t *__restrict__ vin,
+                                                               K *__restrict__ kout, uint32_t *__restrict__ vout, int64_t n,
+                                                               int shift, const uint32_t *__restrict__ hist, int nblocks)
+{
+    __shared__ uint32_t cnt[4][256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int w = 0; w < 4; ++w) cnt[w][threadIdx.x] = 0;
+    __syncthreads();
+    // wave w owns the contiguous 512 keys [base + 512 w, +512), 64 per round
+    const int64_t base = (int64_t)blockIdx.x * RGX_RS_TILE + (int64_t)wave * (64 * RGX_RS_ITEMS);
+    K key[RGX_RS_ITEMS];
+    uint32_t val[RGX_RS_ITEMS];
+    for (int r = 0; r < RGX_RS_ITEMS; ++r) {
+        const int64_t i = base + r * 64 + lane;
+        key[r] = 0;
+        val[r] = 0;
+        if (i < n) {
+            key[r] = kin[i];
+            val[r] = vin[i];
+            atomicAdd(&cnt[wave][(uint32_t)(key[r] >> shift) & 255u], 1u);
+        }
+    }
+    __syncthreads();
+    {
+        const int d = threadIdx.x;
+        uint32_t run = hist[(size_t)d * nblocks + blockIdx.x];
+        for (int w = 0; w < 4; ++w) {
+            const uint32_t c = cnt[w][d];
+            cnt[w][d] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    volatile uint32_t *cur = cnt[wave];
+    for (int r = 0; r < RGX_RS_ITEMS; ++r) {
+        const int64_t i = base + r * 64 + lane;
+        const bool valid = i < n;
+        const uint32_t d = (uint32_t)(key[r] >> shift) & 255u;
+        uint64_t same = __ballot(valid);
+        for (int b = 0; b < 8; ++b) {
+            const bool bit = (d >> b) & 1u;
+            const uint64_t bal = __ballot(bit);
+            same &= bit ? bal : ~bal;
+        }
+        if (valid) {
+            const uint32_t rank = __popcll(same & ((1ull << lane) - 1ull));
+            const uint32_t off = cur[d];
+            kout[off + rank] = key[r];
+            vout[off + rank] = val[r];
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (valid && (same & ((1ull << lane) - 1ull)) == 0) cur[d] += __popcll(same);
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+template <typename K>
+static int radix_sort(K *k0, uint32_t *v0, K *k1, uint32_t *v1, int64_t n, int bits, uint32_t *hist, hipStream_t s)
+{
+    const int nblocks = (int)((n + RGX_RS_TILE - 1) / RGX_RS_TILE);
+    K *ki = k0, *ko = k1;
+    uint32_t *vi = v0, *vo = v1;
+    for (int shift = 0; shift < bits; shift += 8) {
+        hipLaunchKernelGGL(k_rs_hist<K>, dim3(nblocks), dim3(RGX_RS_THREADS), 0, s, ki, n, shift, hist, nblocks);
+        hipLaunchKernelGGL(k_rs_scan, dim3(1), dim3(1024), 0, s, hist, (int64_t)256 * nblocks);
+        hipLaunchKernelGGL(k_rs_scatter<K>, dim3(nblocks), dim3(RGX_RS_THREADS), 0, s, ki, vi, ko, vo, n, shift, hist, nblocks);
+        K *tk = ki; ki = ko; ko = tk;
+        uint32_t *tv = vi; vi = vo; vo = tv;
+    }
+    RGX_LAUNCH_CHECK();
+    return ((bits + 7) / 8) & 1; // 1 when the result ended in (k1, v1)
+}
+
+// ---------------------------------------------------------------------------
+// Leaves, radix tree (Karras 2012), refit, skip links.
+__global__ __launch_bounds__(256) void k_leaves(const float *__restrict__ boxes, const uint32_t *__restrict__ order, int64_t n,
+                                                Node *__restrict__ nodes, int32_t *__restrict__ parent, int32_t *__restrict__ flags)
+{
+    const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    const float *b = boxes + 6 * (int64_t)order[j];
+    Node nd;
+    nd.lo[0] = b[0]; nd.lo[1] = b[1]; nd.lo[2] = b[2];
+    nd.hi[0] = b[3]; nd.hi[1] = b[4]; nd.hi[2] = b[5];
+    nd.left = ~(int32_t)j;
+    nd.skip = -1;
+    nodes[n - 1 + j] = nd;
+    flags[j] = 0;
+    if (j == 0) parent[0] = -1;
+}
+
+__device__ __forceinline__ int delta(const uint64_t *keys, int64_t n, int64_t i, int64_t j)
+{
+    if (j < 0 || j >= n) return -1;
+    const uint64_t a = keys[i], b = keys[j];
+    if (a != b) return __clzll((long long)(a ^ b));
+    return 64 + __clz((int)((uint32_t)i ^ (uint32_t)j));
+}
+
+__global__ __launch_bounds__(256) void k_karras(const uint64_t *__restrict__ keys, int64_t n, Node *__restrict__ nodes,
+                                                int32_t *__restrict__ parent, int32_t *__restrict__ right)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n - 1) return;
+    const int d = delta(keys, n, i, i + 1) - delta(keys, n, i, i - 1) >= 0 ? 1 : -1;
+    const int dmin = delta(keys, n, i, i - d);
+    int64_t lmax = 2;
+    while (delta(keys, n, i, i + lmax * d) > dmin) lmax <<= 1;
+    int64_t l = 0;
+    for (int64_t t = lmax >> 1; t >= 1; t >>= 1)
+        if (delta(keys, n, i, i + (l + t) * d) > dmin) l += t;
+    const int64_t j = i + l * d;
+    const int dnode = delta(keys, n, i, j);
+    int64_t s = 0, t = l;
+    do {
+        t = (t + 1) >> 1;
+        if (delta(keys, n, i, i + (s + t) * d) > dnode) s += t;
+    } while (t > 1);
+    const int64_t gamma = i + s * d + (d < 0 ? -1 : 0);
+    const int64_t lo = i < j ? i : j, hi = i < j ? j : i;
+    const int32_t lc = (int32_t)(lo == gamma ? n - 1 + gamma : gamma);
+    const int32_t rc = (int32_t)(hi == gamma + 1 ? n - 1 + gamma + 1 : gamma + 1);
+    nodes[i].left = lc;
+    right[i] = rc;
+    parent[lc] = (int32_t)i;
+    parent[rc] = (int32_t)i;
+}
+
+__global__ __launch_bounds__(256) void k_refit(int64_t n, Node *nodes, const int32_t *__restrict__ parent,
+                                               const int32_t *__restrict__ right, int32_t *flags)
+{
+    const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= n) return;
+    int32_t node = parent[n - 1 + j];
+    while (node >= 0) {
+        __threadfence();
+        if (atomicAdd(&flags[node], 1) == 0) return; // the sibling subtree is not done yet
+        __threadfence();
+        const Node *a = &nodes[nodes[node].left];
+        const Node *b = &nodes[right[node]];
+        // volatile reads: the children were written by other workgroups during this launch
+        const volatile float *al = a->lo, *ah = a->hi, *bl = b->lo, *bh = b->hi;
+        for (int c = 0; c < 3; ++c) {
+            nodes[node].lo[c] = fminf(al[c], bl[c]);
+            nodes[node].hi[c] = fmaxf(ah[c], bh[c]);
+        }
+        node = parent[node];
+    }
+}
+
+__global__ __launch_bounds__(256) void k_skip_links(int64_t n, Node *__restrict__ nodes, const int32_t *__restrict__ parent,
+                                                    const int32_t *__restrict__ right)
+{
+    const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= 2 * n - 1) return;
+    int32_t cur = (int32_t)id, skip = -1;
+    for (;;) {
+        const int32_t p = parent[cur];
+        if (p < 0) break;
+        if (nodes[p].left == cur) { skip = right[p]; break; }
+        cur = p;
+    }
+    nodes[id].skip = skip;
+}
+
+__global__ void k_mark_built(WsHeader *h) { h->built = 1; }
+
+// ---------------------------------------------------------------------------
+static inline dim3 grid_for(int64_t n, int block) { return dim3((unsigned)((n + block - 1) / block)); }
+
+extern "C" int rgx_aabb(const float *pos, const float *scale, const float *quat, const float *dens, int64_t n,
+                        float sigma_threshold, float *bboxes, float *bb_min, float *bb_max, void *stream)
+{
+    if (n < 0 || (n > 0 && (!pos || !scale || !quat || !dens)) || ((bb_min == nullptr) != (bb_max == nullptr)))
+        return RGX_EINVAL;
+    hipStream_t s = (hipStream_t)stream;
+    int32_t *mn = (int32_t *)bb_min, *mx = (int32_t *)bb_max;
+    if (mn) hipLaunchKernelGGL(k_init_enc, dim3(1), dim3(64), 0, s, mn, mx);
+    if (n > 0)
+        hipLaunchKernelGGL(k_aabb, grid_for(n, 256), dim3(256), 0, s, pos, scale, quat, dens, n, sigma_threshold, bboxes, mn, mx);
+    if (mn) hipLaunchKernelGGL(k_decode_enc, dim3(1), dim3(64), 0, s, mn, mx);
+    RGX_LAUNCH_CHECK();
+    return RGX_OK;
+}
+
+extern "C" int rgx_build_workspace_bytes(int64_t n, size_t *bytes)
+{
+    if (n < 0 || !bytes || n > 0x3fffffff) return RGX_EINVAL;
+    *bytes = rgx_ws_layout(n).total;
+    return RGX_OK;
+}
+
+// Copies caller-supplied boxes into the workspace and reduces the scene bbox.
+__global__ __launch_bounds__(256) void k_take_boxes(const float *__restrict__ in, int64_t n, float *__restrict__ boxes,
+                                                    int32_t *mn_enc, int32_t *mx_enc)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    float b[6] = {INFINITY, INFINITY, INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    if (i < n)
+        for (int a = 0; a < 6; ++a) boxes[6 * i + a] = b[a] = in[6 * i + a];
+    __shared__ float red[4][6];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int a = 0; a < 3; ++a) {
+        const float mn = wave_min(b[a]), mx = wave_max(b[a + 3]);
+        if (lane == 0) { red[wave][a] = mn; red[wave][a + 3] = mx; }
+    }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+        const int a = threadIdx.x;
+        atomicMin(&mn_enc[a], enc_f(fminf(fminf(red[0][a], red[1][a]), fminf(red[2][a], red[3][a]))));
+        atomicMax(&mx_enc[a], enc_f(fmaxf(fmaxf(red[0][a + 3], red[1][a + 3]), fmaxf(red[2][a + 3], red[3][a + 3]))));
+    }
+}
+
+static int build_impl(const float *pos, const float *scale, const float *quat, const float *dens, const float *in_boxes,
+                      int64_t n, float sigma_threshold, void *ws, size_t ws_bytes, void *stream);
+
+extern "C" int rgx_build(const float *pos, const float *scale, const float *quat, const float *dens, int64_t n,
+                         float sigma_threshold, void *ws, size_t ws_bytes, void *stream)
+{
+    if (n > 0 && (!pos || !scale || !quat || !dens)) return RGX_EINVAL;
+    return build_impl(pos, scale, quat, dens, nullptr, n, sigma_threshold, ws, ws_bytes, stream);
+}
+
+extern "C" int rgx_build_aabbs(const float *bboxes, int64_t n, void *ws, size_t ws_bytes, void *stream)
+{
+    if (n > 0 && !bboxes) return RGX_EINVAL;
+    return build_impl(nullptr, nullptr, nullptr, nullptr, bboxes, n, 0.f, ws, ws_bytes, stream);
+}
+
+static int build_impl(const float *pos, const float *scale, const float *quat, const float *dens, const float *in_boxes,
+                      int64_t n, float sigma_threshold, void *ws, size_t ws_bytes, void *stream)
+{
+    if (n < 0 || n > 0x3fffffff || !ws) return RGX_EINVAL;
+    const WsLayout L = rgx_ws_layout(n);
+    if (ws_bytes < L.total || ((uintptr_t)ws & 255u)) return RGX_EWORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    char *w = (char *)ws;
+    WsHeader *hdr = (WsHeader *)(w + L.header);
+    float *boxes = (float *)(w + L.aabb);
+    uint64_t *k0 = (uint64_t *)(w + L.keys0), *k1 = (uint64_t *)(w + L.keys1);
+    uint32_t *v0 = (uint32_t *)(w + L.vals0), *v1 = (uint32_t *)(w + L.vals1);
+    Node *nodes = (Node *)(w + L.nodes);
+    int32_t *parent = (int32_t *)(w + L.parent), *right = (int32_t *)(w + L.right), *flags = (int32_t *)(w + L.flags);
+    uint32_t *hist = (uint32_t *)(w + L.hist);
+
+    void *span = rgx_span_begin(RGX_T_BUILD, s);
+    hipLaunchKernelGGL(k_init_header, dim3(1), dim3(64), 0, s, hdr, n);
+    if (n > 0) {
+        if (in_boxes)
+            hipLaunchKernelGGL(k_take_boxes, grid_for(n, 256), dim3(256), 0, s, in_boxes, n, boxes, hdr->bb_min_enc,
+                               hdr->bb_max_enc);
+        else
+            hipLaunchKernelGGL(k_aabb, grid_for(n, 256), dim3(256), 0, s, pos, scale, quat, dens, n, sigma_threshold, boxes,
+                               hdr->bb_min_enc, hdr->bb_max_enc);
+        hipLaunchKernelGGL(k_finish_bbox, dim3(1), dim3(64), 0, s, hdr, (float *)nullptr, (float *)nullptr);
+        hipLaunchKernelGGL(k_morton63, grid_for(n, 256), dim3(256), 0, s, boxes, n, hdr, k0, v0);
+        RGX_LAUNCH_CHECK();
+        const int r = radix_sort<uint64_t>(k0, v0, k1, v1, n, 64, hist, s);
+        if (r < 0) return r;
+        // 8 passes: the sorted keys / permutation are back in (k0, v0)
+        hipLaunchKernelGGL(k_leaves, grid_for(n, 256), dim3(256), 0, s, boxes, v0, n, nodes, parent, flags);
+        if (n > 1) {
+            hipLaunchKernelGGL(k_karras, grid_for(n - 1, 256), dim3(256), 0, s, k0, n, nodes, parent, right);
+            hipLaunchKernelGGL(k_refit, grid_for(n, 256), dim3(256), 0, s, n, nodes, parent, right, flags);
+        }
+        hipLaunchKernelGGL(k_skip_links, grid_for(2 * n - 1, 256), dim3(256), 0, s, n, nodes, parent, right);
+    }
+    hipLaunchKernelGGL(k_mark_built, dim3(1), dim3(1), 0, s, hdr);
+    rgx_span_end(span, s);
+    RGX_LAUNCH_CHECK();
+    return RGX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Synchronous / small read-backs of a built workspace.
+extern "C" int rgx_scene_bbox(const void *ws, float *host_out6, void *stream)
+{
+    if (!ws || !host_out6) return RGX_EINVAL;
+    const WsHeader *hdr = (const WsHeader *)ws;
+    RGX_HIP(hipMemcpyAsync(host_out6, hdr->bb_min, 6 * sizeof(float), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    RGX_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return RGX_OK;
+}
+
+__global__ __launch_bounds__(256) void k_copy_order(const uint32_t *__restrict__ v, int64_t n, int32_t *__restrict__ out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = (int32_t)v[i];
+}
+
+extern "C" int rgx_build_order(const void *ws, int64_t n, int32_t *order_out, void *stream)
+{
+    if (!ws || n < 0 || (n > 0 && !order_out)) return RGX_EINVAL;
+    if (n == 0) return RGX_OK;
+    const WsLayout L = rgx_ws_layout(n);
+    hipLaunchKernelGGL(k_copy_order, grid_for(n, 256), dim3(256), 0, (hipStream_t)stream,
+                       (const uint32_t *)((const char *)ws + L.vals0), n, order_out);
+    RGX_LAUNCH_CHECK();
+    return RGX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// 30-bit Morton ordering of the point cloud (utils/reordering_utils.py:55-104,
+// classes/point_cloud.py:1017-1024).
+__global__ __launch_bounds__(256) void k_pos_minmax(const float *__restrict__ pos, int64_t n, int32_t *mn_enc, int32_t *mx_enc)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    float b[6] = {INFINITY, INFINITY, INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    if (i < n)
+        for (int a = 0; a < 3; ++a) b[a] = b[a + 3] = pos[3 * i + a];
+    __shared__ float red[4][6];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int a = 0; a < 3; ++a) {
+        const float mn = wave_min(b[a]), mx = wave_max(b[a + 3]);
+        if (lane == 0) { red[wave][a] = mn; red[wave][a + 3] = mx; }
+    }
+    __syncthreads();
+    if (threadIdx.x < 3) {
+        const int a = threadIdx.x;
+        atomicMin(&mn_enc[a], enc_f(fminf(fminf(red[0][a], red[1][a]), fminf(red[2][a], red[3][a]))));
+        atomicMax(&mx_enc[a], enc_f(fmaxf(fmaxf(red[0][a + 3], red[1][a + 3]), fmaxf(red[2][a + 3], red[3][a + 3]))));
+    }
+}
+
+__global__ __launch_bounds__(256) void k_morton30(const float *__restrict__ pos, int64_t n, const float *__restrict__ mn,
+                                                  const float *__restrict__ mx, uint32_t *__restrict__ keys,
+                                                  uint32_t *__restrict__ vals, int64_t *__restrict__ codes)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    uint32_t code = 0;
+    for (int a = 0; a < 3; ++a) {
+        const float scale = 1023.0f / ((mx[a] - mn[a]) + 1e-9f); // reordering_utils.py:73
+        const int32_t q = (int32_t)((pos[3 * i + a] - mn[a]) * scale); // .to(torch.int32): truncation
+        for (int b = 0; b < 10; ++b) code |= (uint32_t)((q >> b) & 1) << (3 * b + a); // reordering_utils.py:98-102
+    }
+    keys[i] = code;
+    vals[i] = (uint32_t)i;
+    if (codes) codes[i] = (int64_t)code;
+}
+
+__global__ __launch_bounds__(256) void k_order64(const uint32_t *__restrict__ v, int64_t n, int64_t *__restrict__ out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = (int64_t)v[i];
+}
+
+struct MortonLayout {
+    size_t enc, keys0, keys1, vals0, vals1, hist, total;
+};
+static inline MortonLayout morton_layout(int64_t n)
+{
+    MortonLayout L;
+    const size_t nn = (size_t)(n > 0 ? n : 1), nblocks = (nn + RGX_RS_TILE - 1) / RGX_RS_TILE;
+    size_t off = 0;
+    L.enc = off;   off = rgx_align_up(off + 8 * sizeof(int32_t), 256);
+    L.keys0 = off; off = rgx_align_up(off + nn * 4, 256);
+    L.keys1 = off; off = rgx_align_up(off + nn * 4, 256);
+    L.vals0 = off; off = rgx_align_up(off + nn * 4, 256);
+    L.vals1 = off; off = rgx_align_up(off + nn * 4, 256);
+    L.hist = off;  off = rgx_align_up(off + 256 * nblocks * 4, 256);
+    L.total = off;
+    return L;
+}
+
+extern "C" int rgx_morton_workspace_bytes(int64_t n, size_t *bytes)
+{
+    if (n < 0 || !bytes || n > 0x3fffffff) return RGX_EINVAL;
+    *bytes = morton_layout(n).total;
+    return RGX_OK;
+}
+
+extern "C" int rgx_morton_order(const float *pos, int64_t n, int64_t *codes, int64_t *order, void *ws, size_t ws_bytes,
+                                void *stream)
+{
+    if (n < 0 || n > 0x3fffffff || !ws || (n > 0 && !pos)) return RGX_EINVAL;
+    const MortonLayout L = morton_layout(n);
+    if (ws_bytes < L.total || ((uintptr_t)ws & 255u)) return RGX_EWORKSPACE;
+    if (n == 0) return RGX_OK;
+    hipStream_t s = (hipStream_t)stream;
+    char *w = (char *)ws;
+    int32_t *mn = (int32_t *)(w + L.enc), *mx = mn + 4;
+    uint32_t *k0 = (uint32_t *)(w + L.keys0), *k1 = (uint32_t *)(w + L.keys1);
+    uint32_t *v0 = (uint32_t *)(w + L.vals0), *v1 = (uint32_t *)(w + L.vals1);
+    hipLaunchKernelGGL(k_init_enc, dim3(1), dim3(64), 0, s, mn, mx);
+    hipLaunchKernelGGL(k_pos_minmax, grid_for(n, 256), dim3(256), 0, s, pos, n, mn, mx);
+    hipLaunchKernelGGL(k_decode_enc, dim3(1), dim3(64), 0, s, mn, mx);
+    hipLaunchKernelGGL(k_morton30, grid_for(n, 256), dim3(256), 0, s, pos, n, (const float *)mn, (const float *)mx, k0, v0, codes);
+    RGX_LAUNCH_CHECK();
+    if (order) {
+        const int r = radix_sort<uint32_t>(k0, v0, k1, v1, n, 32, (uint32_t *)(w + L.hist), s);
+        if (r < 0) return r;
+        hipLaunchKernelGGL(k_order64, grid_for(n, 256), dim3(256), 0, s, v0, n, order);
+        RGX_LAUNCH_CHECK();
+    }
+    return RGX_OK;
+}

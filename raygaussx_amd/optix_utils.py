@@ -1,0 +1,283 @@
+"""Host launch glue with the names and argument meaning of the reference's
+``optix_raycasting/optix_utils.py``, implemented on librgx (HIP, gfx950).
+
+What was an OptiX object in the reference is an inert handle here (context,
+module, program groups, pipeline, SBT): the kernels are compiled ahead of time
+into librgx.so, so those constructors only exist to keep caller code unchanged.
+The acceleration structure is real: an LBVH held in a torch byte tensor.
+"""
+import ctypes as C
+import math
+
+import torch
+
+from . import _lib as L
+
+SIGMA_THRESHOLD = 0.1            # cuda_train/forward/gaussians_aabb.h:5
+TRANSMITTANCE_EPSILON = 1e-3     # cuda_train/forward/gaussians_aabb.h:4
+
+_scratch = {}
+
+
+def _workspace(key, nbytes, device):
+    """Cached byte tensor (grown, never shrunk) -- keeps the hot path free of allocations."""
+    t = _scratch.get((key, device))
+    if t is None or t.numel() < nbytes:
+        t = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        _scratch[(key, device)] = t
+    return t
+
+
+class _Handle:
+    """Stands in for an OptiX context / module / program group / pipeline / SBT."""
+
+    def __init__(self, kind, **kw):
+        self.kind = kind
+        self.__dict__.update(kw)
+
+    cache_enabled = False
+
+
+class AccelerationStructure:
+    """LBVH over the Gaussians' k-sigma boxes (replaces ``ox.AccelerationStructure``)."""
+
+    def __init__(self, n, device):
+        self.n = int(n)
+        self.device = device
+        nbytes = L.size_query(L.lib().rgx_build_workspace_bytes, C.c_int64(self.n))
+        self.ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+    @property
+    def handle(self):
+        return self.ws.data_ptr()
+
+    def build_from_gaussians(self, positions, scales, quaternions, densities):
+        L.check(L.lib().rgx_build(L.ptr(positions), L.ptr(scales), L.ptr(quaternions), L.ptr(densities),
+                                  C.c_int64(self.n), C.c_float(SIGMA_THRESHOLD), L.ptr(self.ws),
+                                  C.c_size_t(self.ws.numel()), L.stream(self.device)))
+        return self
+
+    def build_from_boxes(self, bboxes):
+        L.check(L.lib().rgx_build_aabbs(L.ptr(bboxes), C.c_int64(self.n), L.ptr(self.ws),
+                                        C.c_size_t(self.ws.numel()), L.stream(self.device)))
+        return self
+
+    def update(self, bboxes):
+        return self.build_from_boxes(L.f32(bboxes))
+
+    def scene_bbox(self):
+        out = (C.c_float * 6)()
+        L.check(L.lib().rgx_scene_bbox(L.ptr(self.ws), out, L.stream(self.device)))
+        return list(out[:3]), list(out[3:])
+
+    def order(self):
+        out = torch.empty(self.n, dtype=torch.int32, device=self.device)
+        L.check(L.lib().rgx_build_order(L.ptr(self.ws), C.c_int64(self.n), L.ptr(out), L.stream(self.device)))
+        return out
+
+
+def ellipsoids_bbox_from_quat(quaternions, centers, scales, densities):
+    """optix_utils.py:82-109 -> (bboxes (N,6), bb_min (3), bb_max (3)), device tensors."""
+    q, c, s, d = (L.f32(t) for t in (quaternions, centers, scales, densities))
+    n = c.shape[0]
+    boxes = torch.empty(n, 6, dtype=torch.float32, device=c.device)
+    bb = torch.empty(2, 3, dtype=torch.float32, device=c.device)
+    L.check(L.lib().rgx_aabb(L.ptr(c), L.ptr(s), L.ptr(q), L.ptr(d), C.c_int64(n), C.c_float(SIGMA_THRESHOLD),
+                             L.ptr(boxes), C.c_void_p(bb[0].data_ptr()), C.c_void_p(bb[1].data_ptr()),
+                             L.stream(c.device)))
+    return boxes, bb[0], bb[1]
+
+
+def quaternion_to_rotation(quaternion):
+    """optix_utils.py:111-123: rows of the rotation matrix of (w,x,y,z)."""
+    w, x, y, z = quaternion.unbind(1)
+    L1 = torch.stack([1 - 2 * (y ** 2 + z ** 2), 2 * (x * y - w * z), 2 * (x * z + w * y)], 1)
+    L2 = torch.stack([2 * (x * y + w * z), 1 - 2 * (x ** 2 + z ** 2), 2 * (y * z - w * x)], 1)
+    L3 = torch.stack([2 * (x * z - w * y), 2 * (y * z + w * x), 1 - 2 * (x ** 2 + y ** 2)], 1)
+    return L1, L2, L3
+
+
+def compute_ellipsoids_bbox(centers, scales, L1, L2, L3, densities):
+    """optix_utils.py:125-137 (the legacy box routine scripts/test.py:65-66 calls)."""
+    delta = torch.log((densities / SIGMA_THRESHOLD) ** 2).clamp_min(0).sqrt()
+    ext = torch.stack([torch.linalg.norm(delta[:, None] * scales * Li, dim=1) for Li in (L1, L2, L3)], 1)
+    return torch.cat([centers - ext, centers + ext], 1).float().contiguous()
+
+
+def create_acceleration_structure(ctx, bboxes):
+    """optix_utils.py:139-142: a fresh acceleration structure over (N,6) boxes."""
+    bboxes = L.f32(bboxes)
+    return AccelerationStructure(bboxes.shape[0], bboxes.device).build_from_boxes(bboxes)
+
+
+def update_acceleration_structure(gas, bboxes):
+    """optix_utils.py:144-146 (rebuilds in place; the build is cheap enough not to need a refit path)."""
+    gas.update(bboxes)
+
+
+def create_context(log=None):
+    return _Handle("context", log=log)
+
+
+def create_module(ctx, pipeline_opts, stage, debug_level=None, opt_level=None):
+    if stage not in ("forward", "backward", "test", "gui"):
+        raise ValueError("stage must be 'forward', 'backward', 'test' or 'gui'")
+    if stage == "gui":
+        raise NotImplementedError("the GUI kernel variant is not part of this library")
+    L.lib()  # make a missing library surface here, like a failed module compile would
+    return _Handle("module", stage=stage)
+
+
+def create_program_groups(ctx, module):
+    return [_Handle("program_group", stage=module.stage, index=i) for i in range(5)]
+
+
+def create_pipeline(ctx, program_grps, pipeline_options, debug_level=None):
+    return _Handle("pipeline", stage=program_grps[0].stage)
+
+
+def create_sbt(program_grps):
+    return _Handle("sbt")
+
+
+# ---------------------------------------------------------------------------
+def camera_struct(camera, supersampling=(1, 1)):
+    """Launch constants read from a Camera (optix_utils.py:258-266).  The host copies of the
+    camera tensors are cached on the camera object, so repeated views cost no device sync."""
+    host = getattr(camera, "_rgx_host", None)
+    if host is None:
+        eye = camera.camera_center.detach().reshape(-1).to("cpu", torch.float32).tolist()
+        wvt = camera.world_view_transform.detach().to("cpu", torch.float32)
+        host = (eye, wvt[:3, 0].tolist(), wvt[:3, 1].tolist(), wvt[:3, 2].tolist())
+        try:
+            camera._rgx_host = host
+        except AttributeError:
+            pass
+    c = L.RgxCamera()
+    for a in range(3):
+        c.eye[a], c.u[a], c.v[a], c.w[a] = host[0][a], host[1][a], host[2][a], host[3][a]
+    c.tan_half_fov_x = math.tan(camera.FoVx / 2)
+    c.tan_half_fov_y = math.tan(camera.FoVy / 2)
+    c.principal_x = camera.Px
+    c.principal_y = camera.Py
+    c.width = int(camera.image_width) * int(supersampling[0])
+    c.height = int(camera.image_height) * int(supersampling[1])
+    return c
+
+
+def pack_prims(gas, camera_or_eye, positions, scales, quaternions, densities, rgb, out=None):
+    """The (N,16) PrimData block of optix_utils.py:268-304, in the acceleration structure's order."""
+    n = positions.shape[0]
+    eye = camera_or_eye.eye if isinstance(camera_or_eye, L.RgxCamera) else L.host3(camera_or_eye)
+    if out is None:
+        out = torch.empty(n, 16, dtype=torch.float32, device=positions.device)
+    L.check(L.lib().rgx_pack_prims(L.ptr(gas.ws) if gas is not None else C.c_void_p(0), eye, L.ptr(positions),
+                                   L.ptr(scales), L.ptr(quaternions), L.ptr(densities), L.ptr(rgb), C.c_int64(n),
+                                   C.c_float(SIGMA_THRESHOLD), L.ptr(out), L.stream(positions.device)))
+    return out
+
+
+def _march_ws(n, n_rays, max_prim_slice, device):
+    nbytes = L.size_query(L.lib().rgx_march_workspace_bytes, C.c_int64(n), C.c_int64(n_rays),
+                          C.c_int32(max_prim_slice))
+    return _workspace("march", nbytes, device)
+
+
+def march_forward(gas, cam, prims, dt_step, dynamic_sampling, max_prim_slice, white_background,
+                  t_eps=TRANSMITTANCE_EPSILON, stats=None):
+    n, dev = prims.shape[0], prims.device
+    n_rays = cam.width * cam.height
+    m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), int(bool(white_background)), t_eps)
+    ws = _march_ws(n, n_rays, max_prim_slice, dev)
+    ray_colors = torch.empty(n_rays, 3, dtype=torch.float32, device=dev)
+    L.check(L.lib().rgx_march_forward(L.ptr(gas.ws), C.byref(cam), C.byref(m), L.ptr(prims), C.c_int64(n),
+                                      L.ptr(ray_colors), L.ptr(ws), C.c_size_t(ws.numel()), L.ptr(stats),
+                                      L.stream(dev)))
+    return ray_colors
+
+
+def march_backward(gas, cam, prims, ray_colors, dloss, dt_step, dynamic_sampling, max_prim_slice,
+                   white_background=True, t_eps=TRANSMITTANCE_EPSILON, stats=None):
+    n, dev = prims.shape[0], prims.device
+    n_rays = cam.width * cam.height
+    m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), int(bool(white_background)), t_eps)
+    ws = _march_ws(n, n_rays, max_prim_slice, dev)
+    ddens = torch.empty(n, dtype=torch.float32, device=dev)
+    drgb = torch.empty(n, 3, dtype=torch.float32, device=dev)
+    dpos = torch.empty(n, 3, dtype=torch.float32, device=dev)
+    dscale = torch.empty(n, 3, dtype=torch.float32, device=dev)
+    dquat = torch.empty(n, 4, dtype=torch.float32, device=dev)
+    L.check(L.lib().rgx_march_backward(L.ptr(gas.ws), C.byref(cam), C.byref(m), L.ptr(prims), C.c_int64(n),
+                                       L.ptr(ray_colors), L.ptr(dloss), L.ptr(ddens), L.ptr(drgb), L.ptr(dpos),
+                                       L.ptr(dscale), L.ptr(dquat), L.ptr(ws), C.c_size_t(ws.numel()),
+                                       L.ptr(stats), L.stream(dev)))
+    return ddens, drgb, dpos, dscale, dquat
+
+
+def launch_pipeline_forward(pipeline, sbt, gas, bbox_min, bbox_max, dt_step, dynamic_sampling, camera,
+                            densities, color_features, positions, scales, quaternions, max_prim_slice,
+                            iteration=0, jitter=0, rnd_sample=0, supersampling=(1, 1), white_background=True,
+                            hit_prim_idx=None, t_eps=TRANSMITTANCE_EPSILON, stats=None, return_prims=False):
+    """optix_utils.py:222-322.  ``color_features`` is the per-Gaussian RGB (N,3).  ``bbox_min`` /
+    ``bbox_max`` are accepted for signature compatibility: the acceleration structure already holds the
+    scene box they were computed from.  ``iteration``, ``jitter``, ``rnd_sample`` are dead launch
+    parameters in the reference too; ``hit_prim_idx`` (its per-ray hit scratch) is not needed."""
+    cam = camera_struct(camera, supersampling)
+    prims = pack_prims(gas, cam, L.f32(positions), L.f32(scales), L.f32(quaternions), L.f32(densities),
+                       L.f32(color_features))
+    out = march_forward(gas, cam, prims, dt_step, dynamic_sampling, max_prim_slice, white_background, t_eps, stats)
+    return (out, prims) if return_prims else out
+
+
+def launch_pipeline_test(pipeline, sbt, gas, bbox_min, bbox_max, dt_step, dynamic_sampling, camera, densities,
+                         color_features, positions, scales, quaternions, max_prim_slice, rnd_sample=0,
+                         supersampling=(1, 1), white_background=True, hit_prim_idx=None,
+                         t_eps=TRANSMITTANCE_EPSILON, stats=None):
+    """optix_utils.py:503-601: the inference launch; same kernel as the training forward."""
+    return launch_pipeline_forward(pipeline, sbt, gas, bbox_min, bbox_max, dt_step, dynamic_sampling, camera,
+                                   densities, color_features, positions, scales, quaternions, max_prim_slice,
+                                   rnd_sample=rnd_sample, supersampling=supersampling,
+                                   white_background=white_background, hit_prim_idx=hit_prim_idx, t_eps=t_eps,
+                                   stats=stats)
+
+
+def launch_pipeline_backward(pipeline, sbt, gas, bbox_min, bbox_max, dt_step, dynamic_sampling, camera,
+                             densities, color_features, positions, scales, quaternions, ray_colors,
+                             dloss_dray_colors, max_prim_slice, iteration=0, jitter=0, rnd_sample=0,
+                             supersampling=(1, 1), hit_prim_idx=None, t_eps=TRANSMITTANCE_EPSILON, stats=None,
+                             prims=None):
+    """optix_utils.py:363-500 (+ reduce_temp_grads 325-361): returns densities_grad, color_features_grad
+    (w.r.t. the per-Gaussian RGB), positions_grad, scales_grad, quaternions_grad."""
+    cam = camera_struct(camera, supersampling)
+    if prims is None:
+        prims = pack_prims(gas, cam, L.f32(positions), L.f32(scales), L.f32(quaternions), L.f32(densities),
+                           L.f32(color_features))
+    return march_backward(gas, cam, prims, L.f32(ray_colors), L.f32(dloss_dray_colors), dt_step, dynamic_sampling,
+                          max_prim_slice, True, t_eps, stats)
+
+
+def new_stats(device):
+    """Zeroed device counter block for the ``stats`` arguments."""
+    return torch.zeros(len(L.STATS_FIELDS), dtype=torch.int64, device=device)
+
+
+def read_stats(stats):
+    return dict(zip(L.STATS_FIELDS, stats.tolist()))
+
+
+def first_hit(gas, prims, eye, dirs, tlo, thi):
+    out = torch.empty(dirs.shape[0], dtype=torch.float32, device=dirs.device)
+    L.check(L.lib().rgx_first_hit(L.ptr(gas.ws), L.ptr(prims), C.c_int64(prims.shape[0]), L.host3(eye),
+                                  C.c_int64(dirs.shape[0]), L.ptr(dirs), L.ptr(tlo), L.ptr(thi), L.ptr(out),
+                                  L.stream(dirs.device)))
+    return out
+
+
+def trace_segments(gas, prims, eye, dirs, tlo, thi, cap):
+    n = dirs.shape[0]
+    counts = torch.empty(n, dtype=torch.int32, device=dirs.device)
+    ids = torch.full((n, cap), -1, dtype=torch.int32, device=dirs.device)
+    L.check(L.lib().rgx_trace_segments(L.ptr(gas.ws), L.ptr(prims), C.c_int64(prims.shape[0]), L.host3(eye),
+                                       C.c_int64(n), L.ptr(dirs), L.ptr(tlo), L.ptr(thi), C.c_int32(cap),
+                                       L.ptr(counts), L.ptr(ids), L.stream(dirs.device)))
+    return counts, ids

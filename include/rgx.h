@@ -129,9 +129,9 @@ int rgx_pack_prims(const void *ws, const float *eye, const float *pos, const flo
 
 /* ---- ray march ------------------------------------------------------------ */
 
-/* Scratch for one march launch: the backward's Morton-ordered gradient block
- * and the overflow part of the per-ray hit lists (the reference's hit_prim_idx,
- * optix_utils.py:306). */
+/* Scratch for one march launch: the backward's Morton-ordered gradient block.  (The
+ * reference's per-ray hit scratch hit_prim_idx, optix_utils.py:306, has no counterpart:
+ * hit lists never leave the chip.) */
 int rgx_march_workspace_bytes(int64_t n, int64_t n_rays, int32_t max_prim_slice, size_t *bytes);
 
 /* Replaces launch_pipeline_forward / launch_pipeline_test (optix_utils.py:222-322,
@@ -162,6 +162,13 @@ int rgx_first_hit(const void *ws, const float *prims, int64_t n_prims, const flo
 int rgx_trace_segments(const void *ws, const float *prims, int64_t n_prims, const float *eye, int64_t n,
                        const float *dirs, const float *tlo, const float *thi, int32_t cap,
                        int32_t *counts, int32_t *ids, void *stream);
+
+/* The collect query as the march kernels run it: one 8x8 pixel tile per wavefront, the
+ * tile's Gaussians gathered once and tested per ray.  tlo/thi (W*H) give each pixel's
+ * segment (thi < tlo: pixel idle); counts (W*H) and ids (W*H,cap) as rgx_trace_segments. */
+int rgx_collect_tiles(const void *ws, const RgxCamera *cam, const float *prims, int64_t n_prims,
+                      const float *tlo, const float *thi, int32_t cap, int32_t *counts, int32_t *ids,
+                      void *stream);
 
 /* ---- Morton reordering of the point cloud --------------------------------- */
 

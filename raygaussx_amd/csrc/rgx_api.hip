@@ -51,7 +51,7 @@ void *rgx_span_begin(int id, hipStream_t s)
         delete sp;
         return nullptr;
     }
-    hipEventRecord(sp->a, s);
+    (void)hipEventRecord(sp->a, s);
     return sp;
 }
 
@@ -59,7 +59,7 @@ void rgx_span_end(void *h, hipStream_t s)
 {
     if (!h) return;
     Span *sp = (Span *)h;
-    hipEventRecord(sp->b, s);
+    (void)hipEventRecord(sp->b, s);
     std::lock_guard<std::mutex> lk(g_mu);
     g_spans.push_back(*sp);
     delete sp;
@@ -76,8 +76,8 @@ extern "C" int rgx_timing_reset(void)
 {
     std::lock_guard<std::mutex> lk(g_mu);
     for (Span &sp : g_spans) {
-        hipEventDestroy(sp.a);
-        hipEventDestroy(sp.b);
+        (void)hipEventDestroy(sp.a);
+        (void)hipEventDestroy(sp.b);
     }
     g_spans.clear();
     return RGX_OK;

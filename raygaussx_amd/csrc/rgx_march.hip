@@ -3,18 +3,31 @@
 // (also cuda_test/, byte-identical) and cuda_train/backward/gaussians_aabb.cu, and
 // their launchers (optix_raycasting/optix_utils.py:222-322, 363-500, 503-601).
 //
-// One lane per ray, one 64-lane wavefront per 8x8 pixel tile.  Each ray walks
-// the skip-link BVH once per query (first-hit or collect); a slab's hit list
-// lives in LDS (lane-interleaved, RGX_LDS_HITS entries per ray) and overflows
-// into a global spill area up to max_prim_slice entries.
+// Mapping: one lane per ray, one 64-lane wavefront (= one workgroup) per 8x8 pixel
+// tile, all rays of a tile sharing the camera origin.  Per slab iteration the wave
+//   1. gathers, cooperatively, the Gaussians whose boxes meet the tile's frustum
+//      over the union of the lanes' slab intervals: a 64-wide sweep of the BVH with
+//      the node stack and the candidate table in LDS (one node per lane per step);
+//   2. walks the candidate table in lock step: every lane evaluates the exact hit
+//      predicate for ITS ray and slab (so hit sets are those of a per-ray query),
+//      and the lanes that hit accumulate the candidate's samples.  Candidate data
+//      is wave-uniform, i.e. one 64-byte fetch per wave instead of one per lane;
+//   3. (backward) reduces each candidate's 14 gradient words across the wave with
+//      DPP adds and issues ONE set of atomics per wave and candidate.
+// The first-hit query (once per ray, and after an empty slab) walks the BVH per lane
+// through its skip links.
 #include "rgx_device.h"
 
-#define RGX_LDS_HITS 32
+#define RGX_QCAP 2048      // node stack entries per wave (LDS)
+#define RGX_CCAP 256       // candidate table entries per wave (LDS)
+#define RGX_DFS_MARGIN 192 // above QCAP - margin the sweep pops one node at a time (depth-first)
+#define RGX_LDS_HITS 32    // per-lane list of the stand-alone collect hook
 
 struct MarchParams {
     RgxCamera cam;
     RgxMarch m;
     const Node *nodes;
+    const int32_t *right; // right child of internal node i
     const uint32_t *order;
     const WsHeader *hdr;
     const Prim *prims;
@@ -23,21 +36,8 @@ struct MarchParams {
     const float *fwd_colors; // bwd: forward output (C + T*bg)
     const float *dloss;      // bwd
     float *gbuf;             // bwd: (n,16) gradient block in Morton order
-    int32_t *spill;
-    int32_t spill_cap; // entries per ray beyond RGX_LDS_HITS
     RgxStats *stats;
     int32_t tiles_x, tiles_y;
-};
-
-struct HitList {
-    int32_t *lds;   // &hits[0][lane]
-    int32_t *spill; // this ray's spill row (may be null when spill_cap == 0)
-    __device__ __forceinline__ void put(int j, int32_t v) const
-    {
-        if (j < RGX_LDS_HITS) lds[j * 64] = v;
-        else spill[j - RGX_LDS_HITS] = v;
-    }
-    __device__ __forceinline__ int32_t get(int j) const { return j < RGX_LDS_HITS ? lds[j * 64] : spill[j - RGX_LDS_HITS]; }
 };
 
 struct Counters {
@@ -45,6 +45,39 @@ struct Counters {
     unsigned long long nodes = 0;
 };
 
+// ---------------------------------------------------------------------------
+// wave-wide reductions with DPP (all 64 lanes must be active)
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f(float identity, float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(identity), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+// total in lane 63
+__device__ __forceinline__ float wave_sum_to63(float v)
+{
+    v += dpp_f<0xB1, 0xf>(0.f, v);  // quad_perm [1,0,3,2]
+    v += dpp_f<0x4E, 0xf>(0.f, v);  // quad_perm [2,3,0,1]
+    v += dpp_f<0x141, 0xf>(0.f, v); // row_half_mirror
+    v += dpp_f<0x140, 0xf>(0.f, v); // row_mirror
+    v += dpp_f<0x142, 0xa>(0.f, v); // row_bcast:15 into rows 1,3
+    v += dpp_f<0x143, 0xc>(0.f, v); // row_bcast:31 into rows 2,3
+    return v;
+}
+__device__ __forceinline__ float wave_min_all(float v)
+{
+    v = fminf(v, dpp_f<0xB1, 0xf>(INFINITY, v));
+    v = fminf(v, dpp_f<0x4E, 0xf>(INFINITY, v));
+    v = fminf(v, dpp_f<0x141, 0xf>(INFINITY, v));
+    v = fminf(v, dpp_f<0x140, 0xf>(INFINITY, v));
+    v = fminf(v, dpp_f<0x142, 0xa>(INFINITY, v));
+    v = fminf(v, dpp_f<0x143, 0xc>(INFINITY, v));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+__device__ __forceinline__ float wave_max_all(float v) { return -wave_min_all(-v); }
+
+// ---------------------------------------------------------------------------
+// Per-lane queries through the skip links.
+//
 // First-hit query: optixTrace with SBT offset 0 (gaussians_aabb.cu:234-247, 300-313),
 // __closesthit__ch / __miss__ms_ch (370-380).  Smallest reported t, or -1.
 __device__ float first_hit(const MarchParams &P, f3 o, f3 dir, float tlo, float thi, Counters &cn)
@@ -79,8 +112,19 @@ __device__ float first_hit(const MarchParams &P, f3 o, f3 dir, float tlo, float 
     return best;
 }
 
-// Collect query: optixTrace with SBT offset 1 + __anyhit__ah (gaussians_aabb.cu:282-295,
-// 349-367).  Appends every Gaussian hit in [tlo, thi] (sorted index) until `cap`.
+struct HitList {
+    int32_t *lds;   // &hits[0][lane]
+    int32_t *spill; // entries beyond RGX_LDS_HITS
+    __device__ __forceinline__ void put(int j, int32_t v) const
+    {
+        if (j < RGX_LDS_HITS) lds[j * 64] = v;
+        else spill[j - RGX_LDS_HITS] = v;
+    }
+    __device__ __forceinline__ int32_t get(int j) const { return j < RGX_LDS_HITS ? lds[j * 64] : spill[j - RGX_LDS_HITS]; }
+};
+
+// Collect query, one ray at a time: optixTrace with SBT offset 1 + __anyhit__ah
+// (gaussians_aabb.cu:282-295, 349-367).  Used by the segment test hook.
 __device__ int collect(const MarchParams &P, f3 o, f3 dir, float tlo, float thi, int cap, const HitList &hl, bool &overflow,
                        Counters &cn)
 {
@@ -117,6 +161,121 @@ __device__ int collect(const MarchParams &P, f3 o, f3 dir, float tlo, float thi,
     return p0;
 }
 
+// ---------------------------------------------------------------------------
+// Tile frustum: the four planes through the eye spanned by the tile's corner rays
+// (every pixel ray of the tile lies inside, the image-plane grid being affine) and
+// the shell T0 <= |x - eye| <= T1 (ray directions are unit vectors).  pad (world
+// units) covers the rounding of the exact predicate and of these tests.
+struct Frustum {
+    f3 o;
+    f3 n[4]; // unit normals pointing out of the frustum
+    float t0, t1, pad;
+};
+
+__device__ __forceinline__ f3 cross3(f3 a, f3 b) { return mk3(a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x); }
+
+__device__ __forceinline__ f3 plane_normal(f3 a, f3 b, f3 inside)
+{
+    f3 n = cross3(a, b);
+    n = n * (1.0f / sqrtf(fmaxf(dot3(n, n), 1e-30f)));
+    return dot3(n, inside) > 0.f ? n * -1.0f : n;
+}
+
+__device__ __forceinline__ void frustum_planes(const RgxCamera &cam, int px0, int py0, Frustum &F)
+{
+    const f3 d00 = compute_ray(cam, (unsigned)px0, (unsigned)py0), d10 = compute_ray(cam, (unsigned)(px0 + 7), (unsigned)py0);
+    const f3 d01 = compute_ray(cam, (unsigned)px0, (unsigned)(py0 + 7));
+    const f3 d11 = compute_ray(cam, (unsigned)(px0 + 7), (unsigned)(py0 + 7));
+    const f3 in = (d00 + d10) + (d01 + d11);
+    F.o = mk3(cam.eye[0], cam.eye[1], cam.eye[2]);
+    F.n[0] = plane_normal(d00, d01, in);
+    F.n[1] = plane_normal(d10, d11, in);
+    F.n[2] = plane_normal(d00, d10, in);
+    F.n[3] = plane_normal(d01, d11, in);
+}
+
+__device__ __forceinline__ bool frustum_overlaps(const Frustum &F, float4 a, float4 b)
+{
+    const f3 lo = mk3(a.x - F.o.x, a.y - F.o.y, a.z - F.o.z), hi = mk3(b.x - F.o.x, b.y - F.o.y, b.z - F.o.z);
+    bool out = false;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const f3 n = F.n[k];
+        // box corner closest to the inside of plane k
+        const float d = (n.x * (n.x > 0.f ? lo.x : hi.x) + n.y * (n.y > 0.f ? lo.y : hi.y)) + n.z * (n.z > 0.f ? lo.z : hi.z);
+        out |= d > F.pad;
+    }
+    // distance shell
+    const float nx = fmaxf(fmaxf(lo.x, -hi.x), 0.f), ny = fmaxf(fmaxf(lo.y, -hi.y), 0.f), nz = fmaxf(fmaxf(lo.z, -hi.z), 0.f);
+    const float fx = fmaxf(fabsf(lo.x), fabsf(hi.x)), fy = fmaxf(fabsf(lo.y), fabsf(hi.y)), fz = fmaxf(fabsf(lo.z), fabsf(hi.z));
+    const float dmin2 = (nx * nx + ny * ny) + nz * nz, dmax2 = (fx * fx + fy * fy) + fz * fz;
+    const float near_t = F.t0 - F.pad, far_t = F.t1 + F.pad;
+    out |= near_t > 0.f && dmax2 < near_t * near_t * 0.9999f;
+    out |= dmin2 > far_t * far_t * 1.0001f;
+    return !out;
+}
+
+// Cooperative sweep of the BVH: the node stack is shared by the wave, every step pops
+// up to 64 nodes (one per lane), tests them against the frustum, appends the leaves
+// that pass to the candidate table and pushes the children of the internal nodes that
+// pass.  Returns when the stack is empty (done) or the table might not take another
+// step's leaves; call again to continue with an emptied table.
+struct Sweep {
+    int qn; // stack entries (wave-uniform)
+};
+
+__device__ __forceinline__ void sweep_begin(const MarchParams &P, Sweep &S, int32_t *s_queue)
+{
+    S.qn = P.n > 0 ? 1 : 0;
+    if (threadIdx.x == 0) s_queue[0] = 0;
+    __syncthreads();
+}
+
+__device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int32_t *s_queue, int32_t *s_cand, bool &done,
+                          Counters &cn)
+{
+    const int lane = threadIdx.x;
+    const uint64_t lt = (1ull << lane) - 1ull;
+    const float4 *nodes4 = (const float4 *)P.nodes;
+    const uint32_t n_nodes = (uint32_t)(2 * P.n - 1);
+    int C = 0;
+    while (S.qn > 0 && C + 64 <= RGX_CCAP) {
+        const int m = S.qn > RGX_QCAP - RGX_DFS_MARGIN ? 1 : (S.qn < 64 ? S.qn : 64);
+        const int base = S.qn - m;
+        int32_t node = -1;
+        if (lane < m) node = s_queue[base + lane];
+        __syncthreads();
+        S.qn = base;
+        bool leaf_hit = false, inner_hit = false;
+        int32_t left = 0, right = 0;
+        if ((uint32_t)node < n_nodes) {
+            const float4 a = nodes4[2 * node], b = nodes4[2 * node + 1];
+            if (frustum_overlaps(F, a, b)) {
+                left = __float_as_int(a.w);
+                leaf_hit = left < 0;
+                inner_hit = !leaf_hit;
+                if (inner_hit) right = P.right[node];
+            }
+        }
+        if (lane == 0) cn.nodes += (unsigned)m;
+        const uint64_t bl = __ballot(leaf_hit), bi = __ballot(inner_hit);
+        if (leaf_hit) s_cand[C + __popcll(bl & lt)] = ~left;
+        C += __popcll(bl);
+        if (inner_hit) {
+            const int pos = S.qn + 2 * __popcll(bi & lt);
+            if (pos + 1 < RGX_QCAP) { // cannot fail: see RGX_DFS_MARGIN (tree depth < 128)
+                s_queue[pos] = right;
+                s_queue[pos + 1] = left;
+            }
+        }
+        S.qn += 2 * __popcll(bi);
+        if (S.qn > RGX_QCAP) S.qn = RGX_QCAP;
+        __syncthreads();
+    }
+    done = S.qn == 0;
+    return C;
+}
+
 // Per-hit constants of the sample recurrence (gaussians_aabb.cu:135-164).
 struct HitSetup {
     float power, inc, inc_st, cut;
@@ -140,18 +299,16 @@ __device__ __forceinline__ HitSetup hit_setup(const Prim &p, f3 dir, f3 ray_dir_
     return h;
 }
 
-__device__ __forceinline__ void tile_pixel(const MarchParams &P, int &px, int &py, bool &valid)
+__device__ __forceinline__ bool tile_origin(const MarchParams &P, int &px0, int &py0)
 {
     // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one contiguous
     // band of tiles so its L2 sees one region of the scene.
     const int ntiles = P.tiles_x * P.tiles_y;
     const int per = (gridDim.x + 7) >> 3;
     const int tile = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-    const int lane = threadIdx.x;
-    const int tx = tile % P.tiles_x, ty = tile / P.tiles_x;
-    px = tx * 8 + (lane & 7);
-    py = ty * 8 + (lane >> 3);
-    valid = tile < ntiles && px < P.cam.width && py < P.cam.height;
+    px0 = (tile % P.tiles_x) * 8;
+    py0 = (tile / P.tiles_x) * 8;
+    return tile < ntiles;
 }
 
 __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
@@ -169,105 +326,271 @@ __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
     }
 }
 
+// State of one ray between slab iterations; the slab loop itself is wave-uniform.
+struct RayState {
+    f3 dir;
+    float tenter, texit, tbuffer, T, dt, slab_spacing;
+    bool active;
+};
+
+// Ray set-up up to the first hit: computeRay, scene-bbox slab test, first-hit query
+// (fwd: gaussians_aabb.cu:207-260; bwd: backward/gaussians_aabb.cu:211-254, which divides
+// by the direction where the forward multiplies by its reciprocal).
+template <bool DIVIDE>
+__device__ __forceinline__ void ray_begin(const MarchParams &P, int px, int py, bool valid, RayState &R, Counters &cn)
+{
+    const f3 o = mk3(P.cam.eye[0], P.cam.eye[1], P.cam.eye[2]);
+    R.dir = compute_ray(P.cam, (unsigned)px, (unsigned)py);
+    const float *bmn = P.hdr->bb_min, *bmx = P.hdr->bb_max;
+    float t0x, t1x, t0y, t1y, t0z, t1z;
+    if (DIVIDE) {
+        t0x = (bmn[0] - o.x) / R.dir.x; t1x = (bmx[0] - o.x) / R.dir.x;
+        t0y = (bmn[1] - o.y) / R.dir.y; t1y = (bmx[1] - o.y) / R.dir.y;
+        t0z = (bmn[2] - o.z) / R.dir.z; t1z = (bmx[2] - o.z) / R.dir.z;
+    } else {
+        const f3 inv = mk3(1.0f / R.dir.x, 1.0f / R.dir.y, 1.0f / R.dir.z);
+        t0x = (bmn[0] - o.x) * inv.x; t1x = (bmx[0] - o.x) * inv.x;
+        t0y = (bmn[1] - o.y) * inv.y; t1y = (bmx[1] - o.y) * inv.y;
+        t0z = (bmn[2] - o.z) * inv.z; t1z = (bmx[2] - o.z) * inv.z;
+    }
+    R.tenter = fmaxf(0.0f, fmaxf(fminf(t0x, t1x), fmaxf(fminf(t0y, t1y), fminf(t0z, t1z))));
+    R.texit = fminf(fmaxf(t0x, t1x), fminf(fmaxf(t0y, t1y), fmaxf(t0z, t1z)));
+    R.dt = P.m.dt_step;
+    R.slab_spacing = R.dt * RGX_BUFFER_SIZE;
+    R.T = 1.0f;
+    R.active = false;
+    R.tbuffer = 0.f;
+    if (valid) {
+        const float fh = first_hit(P, o, R.dir, R.tenter, R.texit, cn);
+        if (fh != -1.0f) {
+            cn.rays_hit++;
+            R.tenter = fh;
+            R.active = R.tenter < R.texit;
+            R.tbuffer = R.tenter;
+        }
+    }
+}
+
+// Top of a slab iteration: loop condition, adaptive step (gaussians_aabb.cu:266-276), slab bounds.
+// CLIP: the forward clips the slab to [tenter, texit] (275-276), the backward does not (279-280).
+template <bool CLIP>
+__device__ __forceinline__ bool slab_begin(const MarchParams &P, RayState &R, float &tlo, float &thi)
+{
+    R.active = R.active && R.tbuffer < R.texit && R.T > P.m.t_eps;
+    // a step below one ulp of t cannot advance the ray: stop instead of spinning
+    R.active = R.active && (R.tbuffer + R.slab_spacing > R.tbuffer);
+    if (R.active && P.m.dynamic_sampling) {
+        const float dt_dist = fmaxf(R.tbuffer / 1024.0f, P.m.dt_step);
+        const float coeff = rcbrtf(R.T);
+        R.dt = fminf(dt_dist * coeff, 4.0f * P.m.dt_step);
+        R.slab_spacing = R.dt * RGX_BUFFER_SIZE;
+    }
+    tlo = CLIP ? fmaxf(R.tenter, R.tbuffer) : R.tbuffer;
+    thi = CLIP ? fminf(R.texit, R.tbuffer + R.slab_spacing) : R.tbuffer + R.slab_spacing;
+    return R.active && thi > R.tenter;
+}
+
+// End of a slab iteration for this ray: skip ahead after an empty slab
+// (gaussians_aabb.cu:297-319) or step to the next slab (324).
+__device__ __forceinline__ void slab_end(const MarchParams &P, RayState &R, bool need, int p0, Counters &cn)
+{
+    if (!R.active) return;
+    if (need && p0 == 0) {
+        cn.empty++;
+        R.tbuffer += R.slab_spacing;
+        const float nt = first_hit(P, mk3(P.cam.eye[0], P.cam.eye[1], P.cam.eye[2]), R.dir, R.tbuffer, R.texit, cn);
+        if (nt == -1.0f) R.active = false;
+        else R.tbuffer = nt;
+    } else {
+        R.tbuffer += R.slab_spacing;
+    }
+}
+
+// Exact per-ray hit test of one candidate (the collect query's __intersection__gaussian +
+// __anyhit__ah, gaussians_aabb.cu:36-92, 349-367) with the max_prim_slice cut.
+__device__ __forceinline__ bool lane_hits(const Prim &p, f3 dir, bool need, float tlo, float thi, int cap, int &p0, bool &ov)
+{
+    if (!need || ov) return false;
+    float r1, r2, t;
+    if (!(line_roots(p.pos4, p.inv_inter4, p.quat4, dir, r1, r2) && segment_hit(r1, r2, tlo, thi, t))) return false;
+    if (p0 >= cap) {
+        ov = true; // optixTerminateRay: this ray collects nothing further in this slab
+        return false;
+    }
+    ++p0;
+    return true;
+}
+
+// ---------------------------------------------------------------------------
+// One pass over all candidates of the current slab iteration.
+//
+// pass_filter sweeps the BVH (in as many table-fuls as needed), evaluates the exact
+// predicate per lane and calls body(prim, pid, hit) for every candidate some lane
+// hits.  When the whole candidate set fitted in ONE table it also records each lane's
+// hit bits, so that a later pass over the same slab (second chunk, gradient pass) can
+// replay them with pass_replay instead of sweeping and testing again.
+struct PassState {
+    int n_saved;   // candidates held in the table (valid when single)
+    bool single;   // the last filter pass needed one table only
+};
+
+template <typename Body>
+__device__ __forceinline__ void pass_filter(const MarchParams &P, const Frustum &F, int32_t *s_queue, int32_t *s_cand,
+                                            uint32_t (*s_mask)[64], PassState &ps, bool record, f3 dir, bool run, float tlo,
+                                            float thi, int cap, int &p0, bool &ov, Counters &cn, Body body)
+{
+    const int lane = threadIdx.x;
+    Sweep S;
+    sweep_begin(P, S, s_queue);
+    bool done = false, first = true;
+    ps.single = false;
+    do {
+        const int C = sweep_next(P, S, F, s_queue, s_cand, done, cn);
+        const bool rec = record && first && done;
+        if (first && done) {
+            ps.single = true;
+            ps.n_saved = C;
+        }
+        first = false;
+        uint32_t mask = 0;
+        for (int c = 0; c < C; ++c) {
+            const int pid = __builtin_amdgcn_readfirstlane(s_cand[c]);
+            const Prim p = P.prims[pid];
+            const bool hit = lane_hits(p, dir, run, tlo, thi, cap, p0, ov);
+            if (rec) {
+                mask |= (uint32_t)hit << (c & 31);
+                if ((c & 31) == 31 || c == C - 1) {
+                    s_mask[c >> 5][lane] = mask;
+                    mask = 0;
+                }
+            }
+            if (__ballot(hit)) body(p, pid, hit);
+        }
+    } while (!done);
+}
+
+template <typename Body>
+__device__ __forceinline__ void pass_replay(const MarchParams &P, const int32_t *s_cand, uint32_t (*s_mask)[64],
+                                            const PassState &ps, bool run, Body body)
+{
+    const int lane = threadIdx.x;
+    uint32_t mask = 0;
+    for (int c = 0; c < ps.n_saved; ++c) {
+        if ((c & 31) == 0) mask = s_mask[c >> 5][lane];
+        const bool hit = run && ((mask >> (c & 31)) & 1u);
+        if (__ballot(hit)) {
+            const int pid = __builtin_amdgcn_readfirstlane(s_cand[c]);
+            const Prim p = P.prims[pid];
+            body(p, pid, hit);
+        }
+    }
+}
+
+__device__ __forceinline__ void frustum_range(Frustum &F, bool need, float tlo, float thi)
+{
+    F.t0 = wave_min_all(need ? tlo : INFINITY);
+    F.t1 = wave_max_all(need ? thi : -INFINITY);
+    F.pad = 2.0f * RGX_PAD_REL * fmaxf(F.t1, 1.0f);
+}
+
 // ---------------------------------------------------------------------------
 // Forward: __raygen__rg (gaussians_aabb.cu:205-340), accumulateChunk (112-180),
 // colorBlendingT_chunked (182-203).
 __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
 {
-    __shared__ int32_t hits[RGX_LDS_HITS][64];
-    int px, py;
-    bool valid;
-    tile_pixel(P, px, py, valid);
+    __shared__ int32_t s_queue[RGX_QCAP];
+    __shared__ int32_t s_cand[RGX_CCAP];
+    __shared__ uint32_t s_mask[RGX_CCAP / 32][64];
+    int px0, py0;
+    if (!tile_origin(P, px0, py0)) return; // whole wave
+    const int lane = threadIdx.x;
+    const int px = px0 + (lane & 7), py = py0 + (lane >> 3);
+    const bool valid = px < P.cam.width && py < P.cam.height;
     Counters cn;
-    if (valid) {
-        const int64_t ray = (int64_t)py * P.cam.width + px;
-        const f3 o = mk3(P.cam.eye[0], P.cam.eye[1], P.cam.eye[2]);
-        const f3 dir = compute_ray(P.cam, (unsigned)px, (unsigned)py);
-        const HitList hl = {&hits[0][threadIdx.x], P.spill ? P.spill + ray * P.spill_cap : nullptr};
-        const float bg = P.m.white_background ? 1.0f : 0.0f;
-        float out_r = bg, out_g = bg, out_b = bg;
-        // scene-bbox slab test (gaussians_aabb.cu:212-224)
-        const f3 inv = mk3(1.0f / dir.x, 1.0f / dir.y, 1.0f / dir.z);
-        const float *bmn = P.hdr->bb_min, *bmx = P.hdr->bb_max;
-        const float t0x = (bmn[0] - o.x) * inv.x, t1x = (bmx[0] - o.x) * inv.x;
-        const float t0y = (bmn[1] - o.y) * inv.y, t1y = (bmx[1] - o.y) * inv.y;
-        const float t0z = (bmn[2] - o.z) * inv.z, t1z = (bmx[2] - o.z) * inv.z;
-        float tenter = fmaxf(0.0f, fmaxf(fminf(t0x, t1x), fmaxf(fminf(t0y, t1y), fminf(t0z, t1z))));
-        const float texit = fminf(fmaxf(t0x, t1x), fminf(fmaxf(t0y, t1y), fmaxf(t0z, t1z)));
-        const float dt_base = P.m.dt_step;
-        float dt = dt_base, slab_spacing = dt * RGX_BUFFER_SIZE;
-        const float fh = first_hit(P, o, dir, tenter, texit, cn);
-        if (fh != -1.0f) {
-            cn.rays_hit++;
-            tenter = fh;
-            if (tenter < texit) {
-                float T = 1.0f, Cr = 0.f, Cg = 0.f, Cb = 0.f;
-                float tbuffer = tenter;
-                while (tbuffer < texit && T > P.m.t_eps) {
-                    if (!(tbuffer + slab_spacing > tbuffer)) break; // step below one ulp of t: no progress possible
-                    if (P.m.dynamic_sampling) { // gaussians_aabb.cu:267-272
-                        const float dt_dist = fmaxf(tbuffer / 1024.0f, dt_base);
-                        const float coeff = rcbrtf(T);
-                        dt = fminf(dt_dist * coeff, 4.0f * dt_base);
-                        slab_spacing = dt * RGX_BUFFER_SIZE;
+    Frustum F;
+    frustum_planes(P.cam, px0, py0, F);
+    RayState R;
+    ray_begin<false>(P, px, py, valid, R, cn);
+    const f3 dir = R.dir;
+    const int cap = P.m.max_prim_slice;
+    float Cr = 0.f, Cg = 0.f, Cb = 0.f;
+
+    while (__any(R.active)) {
+        float tlo, thi;
+        const bool need = slab_begin<true>(P, R, tlo, thi);
+        int p0 = 0;
+        bool ov = false;
+        if (__any(need)) {
+            frustum_range(F, need, tlo, thi);
+            const float dt = R.dt;
+            PassState ps = {0, false};
+            float sg[RGX_CHUNK_SIZE], cr[RGX_CHUNK_SIZE], cg[RGX_CHUNK_SIZE], cb[RGX_CHUNK_SIZE];
+            f3 rdt;
+            auto accumulate = [&](const Prim &p, int, bool hit) {
+                if (hit) {
+                    HitSetup hs = hit_setup(p, dir, rdt, dt);
+#pragma unroll
+                    for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
+                        const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
+                        sg[i] = fmaf(p.rgba4.w, gw, sg[i]);
+                        cr[i] = fmaf(p.rgba4.x, gw, cr[i]);
+                        cg[i] = fmaf(p.rgba4.y, gw, cg[i]);
+                        cb[i] = fmaf(p.rgba4.z, gw, cb[i]);
+                        hs.power += hs.inc;
+                        hs.inc += hs.inc_st;
                     }
-                    const float t_min_slab = fmaxf(tenter, tbuffer);
-                    const float t_max_slab = fminf(texit, tbuffer + slab_spacing);
-                    if (t_max_slab > tenter) {
-                        bool ov;
-                        const int p0 = collect(P, o, dir, t_min_slab, t_max_slab, P.m.max_prim_slice, hl, ov, cn);
-                        if (ov) cn.overflow++;
-                        if (p0 == 0) {
-                            cn.empty++;
-                            tbuffer += slab_spacing;
-                            const float nt = first_hit(P, o, dir, tbuffer, texit, cn);
-                            if (nt == -1.0f) break;
-                            tbuffer = nt;
-                            continue;
-                        }
-                        cn.slabs++;
-                        cn.hit_pairs += p0;
-                        for (int base = 0; base < RGX_BUFFER_SIZE && T > P.m.t_eps; base += RGX_CHUNK_SIZE) {
-                            float sg[RGX_CHUNK_SIZE], cr[RGX_CHUNK_SIZE], cg[RGX_CHUNK_SIZE], cb[RGX_CHUNK_SIZE];
-#pragma unroll
-                            for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
-                            const float t_mid = fmaf(dt, (float)base + 0.5f, tbuffer);
-                            const f3 rdt = dir * t_mid;
-                            for (int h = 0; h < p0; ++h) {
-                                const Prim p = P.prims[hl.get(h)];
-                                HitSetup hs = hit_setup(p, dir, rdt, dt);
-#pragma unroll
-                                for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
-                                    const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
-                                    sg[i] = fmaf(p.rgba4.w, gw, sg[i]);
-                                    cr[i] = fmaf(p.rgba4.x, gw, cr[i]);
-                                    cg[i] = fmaf(p.rgba4.y, gw, cg[i]);
-                                    cb[i] = fmaf(p.rgba4.z, gw, cb[i]);
-                                    hs.power += hs.inc;
-                                    hs.inc += hs.inc_st;
-                                }
-                            }
-#pragma unroll
-                            for (int i = 0; i < RGX_CHUNK_SIZE; ++i) { // gaussians_aabb.cu:195-201
-                                const float x = sg[i] * dt;
-                                const float w = __expf(-x);
-                                const float s = dt * ((1.0f - w) / fmaxf(x, 1e-6f));
-                                const float ts = T * s;
-                                Cr = fmaf(ts, cr[i], Cr);
-                                Cg = fmaf(ts, cg[i], Cg);
-                                Cb = fmaf(ts, cb[i], Cb);
-                                T *= w;
-                            }
-                        }
-                    }
-                    tbuffer += slab_spacing;
                 }
-                out_r = Cr + T * bg; out_g = Cg + T * bg; out_b = Cb + T * bg;
+            };
+            auto blend = [&]() { // gaussians_aabb.cu:195-201
+#pragma unroll
+                for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
+                    const float x = sg[i] * dt;
+                    const float w = __expf(-x);
+                    const float s = dt * ((1.0f - w) / fmaxf(x, 1e-6f));
+                    const float ts = R.T * s;
+                    Cr = fmaf(ts, cr[i], Cr);
+                    Cg = fmaf(ts, cg[i], Cg);
+                    Cb = fmaf(ts, cb[i], Cb);
+                    R.T *= w;
+                }
+            };
+            // samples 0..15
+#pragma unroll
+            for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
+            rdt = dir * fmaf(dt, 0.5f, R.tbuffer);
+            pass_filter(P, F, s_queue, s_cand, s_mask, ps, true, dir, need, tlo, thi, cap, p0, ov, cn, accumulate);
+            const bool has = need && p0 > 0;
+            if (has) blend();
+            // samples 16..31, only for rays still above the transmittance floor (gaussians_aabb.cu:190)
+            const bool run = has && R.T > P.m.t_eps;
+            if (__any(run)) {
+#pragma unroll
+                for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
+                rdt = dir * fmaf(dt, 16.5f, R.tbuffer);
+                if (ps.single) {
+                    pass_replay(P, s_cand, s_mask, ps, run, accumulate);
+                } else {
+                    int q0 = 0;
+                    bool qov = false;
+                    PassState ps2 = {0, false};
+                    pass_filter(P, F, s_queue, s_cand, s_mask, ps2, false, dir, run, tlo, thi, cap, q0, qov, cn, accumulate);
+                }
+                if (run) blend();
             }
+            if (has) {
+                cn.slabs++;
+                cn.hit_pairs += p0;
+            }
+            if (ov) cn.overflow++;
         }
-        P.ray_colors[3 * ray] = out_r;
-        P.ray_colors[3 * ray + 1] = out_g;
-        P.ray_colors[3 * ray + 2] = out_b;
+        slab_end(P, R, need, p0, cn);
+    }
+    if (valid) {
+        const float bg = P.m.white_background ? 1.0f : 0.0f;
+        const int64_t ray = (int64_t)py * P.cam.width + px;
+        P.ray_colors[3 * ray] = Cr + R.T * bg;
+        P.ray_colors[3 * ray + 1] = Cg + R.T * bg;
+        P.ray_colors[3 * ray + 2] = Cb + R.T * bg;
     }
     flush_stats(P.stats, cn);
 }
@@ -288,181 +611,189 @@ __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
 //   the sample point x_k = x_c + u_k dt dir (u_k = k - 15.5) is affine in k.
 // So the inner loop carries three moments (sum y, sum y u, sum y u^2) instead of
 // nineteen running sums; the `power < k^2` mask follows the reference's 32-step
-// recurrence exactly.
+// recurrence exactly.  The 14 gradient words of a candidate are summed over the
+// lanes that hit it before they reach memory.
 __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
 {
-    __shared__ int32_t hits[RGX_LDS_HITS][64];
-    int px, py;
-    bool valid;
-    tile_pixel(P, px, py, valid);
+    __shared__ int32_t s_queue[RGX_QCAP];
+    __shared__ int32_t s_cand[RGX_CCAP];
+    __shared__ uint32_t s_mask[RGX_CCAP / 32][64];
+    int px0, py0;
+    if (!tile_origin(P, px0, py0)) return; // whole wave
+    const int lane = threadIdx.x;
+    const int px = px0 + (lane & 7), py = py0 + (lane >> 3);
+    const bool valid = px < P.cam.width && py < P.cam.height;
     Counters cn;
+    Frustum F;
+    frustum_planes(P.cam, px0, py0, F);
+    RayState R;
+    ray_begin<true>(P, px, py, valid, R, cn);
+    const f3 dir = R.dir;
+    const int cap = P.m.max_prim_slice;
+    f3 g = mk3(0.f, 0.f, 0.f);
+    float D = 0.f;
     if (valid) {
         const int64_t ray = (int64_t)py * P.cam.width + px;
-        const f3 o = mk3(P.cam.eye[0], P.cam.eye[1], P.cam.eye[2]);
-        const f3 dir = compute_ray(P.cam, (unsigned)px, (unsigned)py);
-        const HitList hl = {&hits[0][threadIdx.x], P.spill ? P.spill + ray * P.spill_cap : nullptr};
-        // backward/gaussians_aabb.cu:222-228 divides by the direction
-        const float *bmn = P.hdr->bb_min, *bmx = P.hdr->bb_max;
-        const float t0x = (bmn[0] - o.x) / dir.x, t1x = (bmx[0] - o.x) / dir.x;
-        const float t0y = (bmn[1] - o.y) / dir.y, t1y = (bmx[1] - o.y) / dir.y;
-        const float t0z = (bmn[2] - o.z) / dir.z, t1z = (bmx[2] - o.z) / dir.z;
-        float tenter = fmaxf(0.0f, fmaxf(fminf(t0x, t1x), fmaxf(fminf(t0y, t1y), fminf(t0z, t1z))));
-        const float texit = fminf(fmaxf(t0x, t1x), fminf(fmaxf(t0y, t1y), fmaxf(t0z, t1z)));
-        const float dt_base = P.m.dt_step;
-        float dt = dt_base, slab_spacing = dt * RGX_BUFFER_SIZE;
-        const float fh = first_hit(P, o, dir, tenter, texit, cn);
-        if (fh != -1.0f && fh < texit) {
-            tenter = fh;
-            float tbuffer = tenter, T = 1.0f;
-            const f3 g = mk3(P.dloss[3 * ray], P.dloss[3 * ray + 1], P.dloss[3 * ray + 2]);
-            float D = dot3(g, mk3(P.fwd_colors[3 * ray], P.fwd_colors[3 * ray + 1], P.fwd_colors[3 * ray + 2]));
-            while (tbuffer < texit && T > P.m.t_eps) {
-                if (!(tbuffer + slab_spacing > tbuffer)) break; // step below one ulp of t: no progress possible
-                if (P.m.dynamic_sampling) {
-                    const float dt_dist = fmaxf(tbuffer / 1024.0f, dt_base);
-                    const float coeff = rcbrtf(T);
-                    dt = fminf(dt_dist * coeff, 4.0f * dt_base);
-                    slab_spacing = dt * RGX_BUFFER_SIZE;
+        g = mk3(P.dloss[3 * ray], P.dloss[3 * ray + 1], P.dloss[3 * ray + 2]);
+        D = dot3(g, mk3(P.fwd_colors[3 * ray], P.fwd_colors[3 * ray + 1], P.fwd_colors[3 * ray + 2]));
+    }
+
+    while (__any(R.active)) {
+        float tlo, thi;
+        const bool need = slab_begin<false>(P, R, tlo, thi);
+        int p0 = 0;
+        bool ov = false;
+        if (__any(need)) {
+            frustum_range(F, need, tlo, thi);
+            const float dt = R.dt, tbuffer = R.tbuffer;
+            PassState ps = {0, false};
+            // (1) s_k and g.c~_k  -> PA, PB
+            float PA[RGX_BUFFER_SIZE], PB[RGX_BUFFER_SIZE];
+#pragma unroll
+            for (int i = 0; i < RGX_BUFFER_SIZE; ++i) PA[i] = PB[i] = 0.f;
+            const f3 rdt0 = dir * fmaf(dt, 0.5f, tbuffer);
+            const f3 rdt1 = dir * fmaf(dt, 16.5f, tbuffer);
+            auto densities = [&](const Prim &p, int, bool hit) {
+                if (hit) {
+                    const float ddc = dot3(g, mk3(p.rgba4.x, p.rgba4.y, p.rgba4.z));
+                    HitSetup hs = hit_setup(p, dir, rdt0, dt);
+#pragma unroll
+                    for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
+                        const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
+                        PA[i] = fmaf(p.rgba4.w, gw, PA[i]);
+                        PB[i] = fmaf(ddc, gw, PB[i]);
+                        hs.power += hs.inc;
+                        hs.inc += hs.inc_st;
+                    }
+                    hs = hit_setup(p, dir, rdt1, dt);
+#pragma unroll
+                    for (int i = RGX_CHUNK_SIZE; i < RGX_BUFFER_SIZE; ++i) {
+                        const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
+                        PA[i] = fmaf(p.rgba4.w, gw, PA[i]);
+                        PB[i] = fmaf(ddc, gw, PB[i]);
+                        hs.power += hs.inc;
+                        hs.inc += hs.inc_st;
+                    }
                 }
-                const float t_min_slab = tbuffer; // unclipped: backward/gaussians_aabb.cu:279-280
-                const float t_max_slab = tbuffer + slab_spacing;
-                if (t_max_slab > tenter) {
-                    bool ov;
-                    const int p0 = collect(P, o, dir, t_min_slab, t_max_slab, P.m.max_prim_slice, hl, ov, cn);
-                    if (ov) cn.overflow++;
-                    if (p0 == 0) {
-                        tbuffer += slab_spacing;
-                        const float nt = first_hit(P, o, dir, tbuffer, texit, cn);
-                        if (nt == -1.0f) break;
-                        tbuffer = nt;
-                        continue;
-                    }
-                    cn.slabs++;
-                    cn.hit_pairs += p0;
-                    // (1) s_k and g.c~_k  -> PA, PB
-                    float PA[RGX_BUFFER_SIZE], PB[RGX_BUFFER_SIZE];
+            };
+            pass_filter(P, F, s_queue, s_cand, s_mask, ps, true, dir, need, tlo, thi, cap, p0, ov, cn, densities);
+            const bool has = need && p0 > 0;
+            // (2) prefix: PA <- a_k, PB <- (T_k e_k - D_k) dt - a_k e_k   (so X_k = PB + PA * g.c_i);
+            // it always covers all 32 samples (330-352)
+            float T_after = R.T, D_after = D;
+            float T_mid = R.T; // transmittance at the chunk boundary: gates the second chunk (398)
+            if (has) {
 #pragma unroll
-                    for (int i = 0; i < RGX_BUFFER_SIZE; ++i) PA[i] = PB[i] = 0.f;
-                    const f3 rdt0 = dir * fmaf(dt, 0.5f, tbuffer);
-                    const f3 rdt1 = dir * fmaf(dt, 16.5f, tbuffer);
-                    for (int h = 0; h < p0; ++h) {
-                        const Prim p = P.prims[hl.get(h)];
-                        const float ddc = dot3(g, mk3(p.rgba4.x, p.rgba4.y, p.rgba4.z));
-                        HitSetup hs = hit_setup(p, dir, rdt0, dt);
+                for (int i = 0; i < RGX_BUFFER_SIZE; ++i) {
+                    if (i == RGX_CHUNK_SIZE) T_mid = T_after;
+                    const float sd = PA[i];
+                    const float inv_d = sd > 0.0f ? 1.0f / sd : 0.0f;
+                    const float e = PB[i] * inv_d;
+                    const float w = __expf(-sd * dt);
+                    const float a = T_after * (1.0f - w) * inv_d;
+                    PA[i] = a;
+                    PB[i] = (T_after * e - D_after) * dt - a * e;
+                    D_after -= T_after * (1.0f - w) * e;
+                    T_after *= w;
+                }
+            }
+            const bool use_second = T_mid > P.m.t_eps;
+            // (3) per candidate: moments per lane, wave sum, one set of atomics
+            const f3 xdir_c = dir * fmaf(dt, 16.0f, tbuffer); // slab centre: t_c = tbuffer + 16 dt
+            auto gradients = [&](const Prim &p, int pid, bool hit) {
+                float out[14];
 #pragma unroll
-                        for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
-                            const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
-                            PA[i] = fmaf(p.rgba4.w, gw, PA[i]);
-                            PB[i] = fmaf(ddc, gw, PB[i]);
-                            hs.power += hs.inc;
-                            hs.inc += hs.inc_st;
-                        }
-                        hs = hit_setup(p, dir, rdt1, dt);
-#pragma unroll
-                        for (int i = RGX_CHUNK_SIZE; i < RGX_BUFFER_SIZE; ++i) {
-                            const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
-                            PA[i] = fmaf(p.rgba4.w, gw, PA[i]);
-                            PB[i] = fmaf(ddc, gw, PB[i]);
-                            hs.power += hs.inc;
-                            hs.inc += hs.inc_st;
-                        }
-                    }
-                    // (2) prefix: PA <- a_k, PB <- (T_k e_k - D_k) dt - a_k e_k   (so X_k = PB + PA * g.c_i)
-                    float T_after = T, D_after = D;
-                    // the prefix always covers all 32 samples (330-352)
-                    float T_mid = T; // transmittance at the chunk boundary: gates the second chunk (398)
+                for (int c = 0; c < 14; ++c) out[c] = 0.f;
+                if (hit) {
+                    const float k = p.inv_inter4.w;
+                    const f3 inv_s = mk3(p.inv_inter4.x * k, p.inv_inter4.y * k, p.inv_inter4.z * k);
+                    const float cut = k * k;
+                    f3 U, V, W;
+                    quat_to_cols(p.quat4, U, V, W);
+                    const float rho = p.rgba4.w;
+                    const float dcg = dot3(mk3(p.rgba4.x, p.rgba4.y, p.rgba4.z), g) / rho;
+                    // mask recurrence exactly as backward/gaussians_aabb.cu:375-396, 437-438
+                    const f3 Us = U * inv_s.x, Vs = V * inv_s.y, Ws = W * inv_s.z;
+                    const f3 M1 = mk3(Us.x, Vs.x, Ws.x), M2 = mk3(Us.y, Vs.y, Ws.y), M3 = mk3(Us.z, Vs.z, Ws.z);
+                    const f3 prel = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
+                    const f3 x0 = prel + dir * (tbuffer + 0.5f * dt);
+                    const f3 Mx0 = (M1 * x0.x + M2 * x0.y) + M3 * x0.z;
+                    const f3 Md = (M1 * dir.x + M2 * dir.y) + M3 * dir.z;
+                    const float Md2 = dot3(Md, Md);
+                    const float Md_dt_2 = (dt * dt) * Md2;
+                    float power = dot3(Mx0, Mx0);
+                    float inc = Md_dt_2 + 2.0f * dot3(Mx0, Md) * dt;
+                    const float inc_st = 2.0f * Md_dt_2;
+                    float s0 = 0.f, s1 = 0.f, s2 = 0.f, gc = 0.f;
 #pragma unroll
                     for (int i = 0; i < RGX_BUFFER_SIZE; ++i) {
-                        if (i == RGX_CHUNK_SIZE) T_mid = T_after;
-                        const float sd = PA[i];
-                        const float inv_d = sd > 0.0f ? 1.0f / sd : 0.0f;
-                        const float e = PB[i] * inv_d;
-                        const float w = __expf(-sd * dt);
-                        const float a = T_after * (1.0f - w) * inv_d;
-                        PA[i] = a;
-                        PB[i] = (T_after * e - D_after) * dt - a * e;
-                        D_after -= T_after * (1.0f - w) * e;
-                        T_after *= w;
+                        const bool on = power < cut && (i < RGX_CHUNK_SIZE || use_second);
+                        const float wd = on ? __expf(-0.5f * power) : 0.0f;
+                        const float y = fmaf(PA[i], dcg, PB[i]) * wd;
+                        const float u = (float)i - 15.5f;
+                        s0 += y;
+                        s1 = fmaf(y, u, s1);
+                        s2 = fmaf(y, u * u, s2);
+                        gc = fmaf(wd, PA[i], gc);
+                        power += inc;
+                        inc += inc_st;
                     }
-                    const bool use_second = T_mid > P.m.t_eps;
-                    // (3) per hit
-                    const f3 xdir_c = dir * fmaf(dt, 16.0f, tbuffer); // slab centre: t_c = tbuffer + 16 dt
-                    for (int h = 0; h < p0; ++h) {
-                        const int32_t pid = hl.get(h);
-                        const Prim p = P.prims[pid];
-                        const float k = p.inv_inter4.w;
-                        const f3 inv_s = mk3(p.inv_inter4.x * k, p.inv_inter4.y * k, p.inv_inter4.z * k);
-                        const float cut = k * k;
-                        f3 U, V, W;
-                        quat_to_cols(p.quat4, U, V, W);
-                        const float rho = p.rgba4.w;
-                        const float dcg = dot3(mk3(p.rgba4.x, p.rgba4.y, p.rgba4.z), g) / rho;
-                        // mask recurrence exactly as backward/gaussians_aabb.cu:375-396, 437-438
-                        const f3 Us = U * inv_s.x, Vs = V * inv_s.y, Ws = W * inv_s.z;
-                        const f3 M1 = mk3(Us.x, Vs.x, Ws.x), M2 = mk3(Us.y, Vs.y, Ws.y), M3 = mk3(Us.z, Vs.z, Ws.z);
-                        const f3 prel = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
-                        const f3 x0 = prel + dir * (tbuffer + 0.5f * dt);
-                        const f3 Mx0 = (M1 * x0.x + M2 * x0.y) + M3 * x0.z;
-                        const f3 Md = (M1 * dir.x + M2 * dir.y) + M3 * dir.z;
-                        const float Md2 = dot3(Md, Md);
-                        const float Md_dt_2 = (dt * dt) * Md2;
-                        float power = dot3(Mx0, Mx0);
-                        float inc = Md_dt_2 + 2.0f * dot3(Mx0, Md) * dt;
-                        const float inc_st = 2.0f * Md_dt_2;
-                        float s0 = 0.f, s1 = 0.f, s2 = 0.f, gc = 0.f;
-#pragma unroll
-                        for (int i = 0; i < RGX_BUFFER_SIZE; ++i) {
-                            const bool on = power < cut && (i < RGX_CHUNK_SIZE || use_second);
-                            const float wd = on ? __expf(-0.5f * power) : 0.0f;
-                            const float y = fmaf(PA[i], dcg, PB[i]) * wd;
-                            const float u = (float)i - 15.5f;
-                            s0 += y;
-                            s1 = fmaf(y, u, s1);
-                            s2 = fmaf(y, u * u, s2);
-                            gc = fmaf(wd, PA[i], gc);
-                            power += inc;
-                            inc += inc_st;
-                        }
-                        // moments -> gradients.  x_k = xc + u_k dt dir, (Mx)_k = Mxc + u_k dt Md
-                        const f3 xc = prel + xdir_c;
-                        const f3 Mxc = (M1 * xc.x + M2 * xc.y) + M3 * xc.z;
-                        const float m1 = s1 * dt, m2 = s2 * (dt * dt);
-                        // sum y (Mx)
-                        const f3 Vy = Mxc * s0 + Md * m1;
-                        // sum y (Mx)_a^2
-                        const f3 Sy = mk3(fmaf(Mxc.x * Mxc.x, s0, fmaf(2.0f * Mxc.x * Md.x, m1, Md.x * Md.x * m2)),
-                                          fmaf(Mxc.y * Mxc.y, s0, fmaf(2.0f * Mxc.y * Md.y, m1, Md.y * Md.y * m2)),
-                                          fmaf(Mxc.z * Mxc.z, s0, fmaf(2.0f * Mxc.z * Md.z, m1, Md.z * Md.z * m2)));
-                        // Q_a = sum y x (Mx)_a  (a vector per row a)
-                        const f3 Qx = (xc * (Mxc.x * s0) + (xc * Md.x + dir * Mxc.x) * m1) + dir * (Md.x * m2);
-                        const f3 Qy = (xc * (Mxc.y * s0) + (xc * Md.y + dir * Mxc.y) * m1) + dir * (Md.y * m2);
-                        const f3 Qz = (xc * (Mxc.z * s0) + (xc * Md.z + dir * Mxc.z) * m1) + dir * (Md.z * m2);
-                        float out[14];
-                        out[0] = s0;                                  // d density
-                        const float gcol = gc * rho;
-                        out[1] = g.x * gcol; out[2] = g.y * gcol; out[3] = g.z * gcol; // d rgb
-                        out[4] = rho * dot3(M1, Vy); out[5] = rho * dot3(M2, Vy); out[6] = rho * dot3(M3, Vy); // d position
-                        out[7] = rho * Sy.x * inv_s.x; out[8] = rho * Sy.y * inv_s.y; out[9] = rho * Sy.z * inv_s.z; // d scale
-                        const f3 d1 = Qx * (-rho * inv_s.x), d2 = Qy * (-rho * inv_s.y), d3 = Qz * (-rho * inv_s.z); // d R columns
-                        const float qx = p.quat4.x, qy = p.quat4.y, qz = p.quat4.z, qw = p.quat4.w;
-                        // backward/gaussians_aabb.cu:469-481
-                        out[10] = 2 * qw * d1.y - 2 * qz * d1.z - 2 * qw * d2.x + 2 * qy * d2.z + 2 * qz * d3.x - 2 * qy * d3.y;
-                        out[11] = 2 * qz * d1.y + 2 * qw * d1.z + 2 * qz * d2.x - 4 * qy * d2.y + 2 * qx * d2.z + 2 * qw * d3.x -
-                                  2 * qx * d3.y - 4 * qy * d3.z;
-                        out[12] = -4 * qz * d1.x + 2 * qy * d1.y - 2 * qx * d1.z + 2 * qy * d2.x + 2 * qw * d2.z + 2 * qx * d3.x +
-                                  2 * qw * d3.y - 4 * qz * d3.z;
-                        out[13] = -4 * qw * d1.x + 2 * qx * d1.y + 2 * qy * d1.z - 2 * qx * d2.x - 4 * qw * d2.y + 2 * qz * d2.z +
-                                  2 * qy * d3.x + 2 * qz * d3.y;
-                        float *dst = P.gbuf + (int64_t)pid * 16;
-#pragma unroll
-                        for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, out[c]);
-                    }
-                    D = D_after;
-                    T = T_after;
+                    // moments -> gradients.  x_k = xc + u_k dt dir, (Mx)_k = Mxc + u_k dt Md
+                    const f3 xc = prel + xdir_c;
+                    const f3 Mxc = (M1 * xc.x + M2 * xc.y) + M3 * xc.z;
+                    const float m1 = s1 * dt, m2 = s2 * (dt * dt);
+                    const f3 Vy = Mxc * s0 + Md * m1; // sum y (Mx)
+                    const f3 Sy = mk3(fmaf(Mxc.x * Mxc.x, s0, fmaf(2.0f * Mxc.x * Md.x, m1, Md.x * Md.x * m2)),
+                                      fmaf(Mxc.y * Mxc.y, s0, fmaf(2.0f * Mxc.y * Md.y, m1, Md.y * Md.y * m2)),
+                                      fmaf(Mxc.z * Mxc.z, s0, fmaf(2.0f * Mxc.z * Md.z, m1, Md.z * Md.z * m2))); // sum y (Mx)_a^2
+                    // Q_a = sum y x (Mx)_a  (one vector per row a of M)
+                    const f3 Qx = (xc * (Mxc.x * s0) + (xc * Md.x + dir * Mxc.x) * m1) + dir * (Md.x * m2);
+                    const f3 Qy = (xc * (Mxc.y * s0) + (xc * Md.y + dir * Mxc.y) * m1) + dir * (Md.y * m2);
+                    const f3 Qz = (xc * (Mxc.z * s0) + (xc * Md.z + dir * Mxc.z) * m1) + dir * (Md.z * m2);
+                    out[0] = s0; // d density
+                    const float gcol = gc * rho;
+                    out[1] = g.x * gcol; out[2] = g.y * gcol; out[3] = g.z * gcol;                         // d rgb
+                    out[4] = rho * dot3(M1, Vy); out[5] = rho * dot3(M2, Vy); out[6] = rho * dot3(M3, Vy); // d position
+                    out[7] = rho * Sy.x * inv_s.x; out[8] = rho * Sy.y * inv_s.y; out[9] = rho * Sy.z * inv_s.z; // d scale
+                    const f3 d1 = Qx * (-rho * inv_s.x), d2 = Qy * (-rho * inv_s.y), d3 = Qz * (-rho * inv_s.z); // d R columns
+                    const float qx = p.quat4.x, qy = p.quat4.y, qz = p.quat4.z, qw = p.quat4.w;
+                    // backward/gaussians_aabb.cu:469-481
+                    out[10] = 2 * qw * d1.y - 2 * qz * d1.z - 2 * qw * d2.x + 2 * qy * d2.z + 2 * qz * d3.x - 2 * qy * d3.y;
+                    out[11] = 2 * qz * d1.y + 2 * qw * d1.z + 2 * qz * d2.x - 4 * qy * d2.y + 2 * qx * d2.z + 2 * qw * d3.x -
+                              2 * qx * d3.y - 4 * qy * d3.z;
+                    out[12] = -4 * qz * d1.x + 2 * qy * d1.y - 2 * qx * d1.z + 2 * qy * d2.x + 2 * qw * d2.z + 2 * qx * d3.x +
+                              2 * qw * d3.y - 4 * qz * d3.z;
+                    out[13] = -4 * qw * d1.x + 2 * qx * d1.y + 2 * qy * d1.z - 2 * qx * d2.x - 4 * qw * d2.y + 2 * qz * d2.z +
+                              2 * qy * d3.x + 2 * qz * d3.y;
                 }
-                tbuffer += slab_spacing;
+                // sum over the lanes that hit this Gaussian, then one lane adds to memory
+#pragma unroll
+                for (int c = 0; c < 14; ++c) out[c] = wave_sum_to63(out[c]);
+                if (lane == 63) {
+                    float *dst = P.gbuf + (int64_t)pid * 16;
+#pragma unroll
+                    for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, out[c]);
+                }
+            };
+            if (__any(has)) {
+                if (ps.single) {
+                    pass_replay(P, s_cand, s_mask, ps, has, gradients);
+                } else {
+                    int q0 = 0;
+                    bool qov = false;
+                    PassState ps2 = {0, false};
+                    pass_filter(P, F, s_queue, s_cand, s_mask, ps2, false, dir, has, tlo, thi, cap, q0, qov, cn, gradients);
+                }
             }
+            if (has) {
+                D = D_after;
+                R.T = T_after;
+                cn.slabs++;
+                cn.hit_pairs += p0;
+            }
+            if (ov) cn.overflow++;
         }
+        slab_end(P, R, need, p0, cn);
     }
     flush_stats(P.stats, cn);
 }
@@ -518,28 +849,59 @@ __global__ __launch_bounds__(64) void k_trace_segments(const MarchParams P, f3 o
     counts[r] = ov ? -p0 : p0;
 }
 
+
+// Test hook for the cooperative collect: per pixel a segment [tlo, thi] (thi < tlo = lane idle);
+// writes each ray's hit count (negated when cut at cap) and the INPUT indices of its hits.
+__global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const float *__restrict__ seg_lo,
+                                                      const float *__restrict__ seg_hi, int cap, int32_t *__restrict__ counts,
+                                                      int32_t *__restrict__ ids)
+{
+    __shared__ int32_t s_queue[RGX_QCAP];
+    __shared__ int32_t s_cand[RGX_CCAP];
+    __shared__ uint32_t s_mask[RGX_CCAP / 32][64];
+    int px0, py0;
+    if (!tile_origin(P, px0, py0)) return;
+    const int lane = threadIdx.x;
+    const int px = px0 + (lane & 7), py = py0 + (lane >> 3);
+    const bool valid = px < P.cam.width && py < P.cam.height;
+    const int64_t ray = (int64_t)py * P.cam.width + px;
+    Counters cn;
+    Frustum F;
+    frustum_planes(P.cam, px0, py0, F);
+    const f3 dir = compute_ray(P.cam, (unsigned)px, (unsigned)py);
+    const float tlo = valid ? seg_lo[ray] : 1.f, thi = valid ? seg_hi[ray] : 0.f;
+    const bool need = valid && thi >= tlo;
+    int p0 = 0;
+    bool ov = false;
+    if (__any(need)) {
+        frustum_range(F, need, tlo, thi);
+        PassState ps = {0, false};
+        auto record = [&](const Prim &, int pid, bool hit) {
+            if (hit) ids[ray * cap + (p0 - 1)] = (int32_t)P.order[pid];
+        };
+        pass_filter(P, F, s_queue, s_cand, s_mask, ps, false, dir, need, tlo, thi, cap, p0, ov, cn, record);
+    }
+    if (valid) counts[ray] = ov ? -p0 : p0;
+}
+
 // ---------------------------------------------------------------------------
 static inline dim3 grid_for(int64_t n, int block) { return dim3((unsigned)((n + block - 1) / block)); }
 
 struct MarchWs {
-    size_t gbuf, spill, total;
-    int32_t spill_cap;
+    size_t gbuf, total;
 };
-static inline MarchWs march_ws_layout(int64_t n, int64_t n_rays, int32_t max_prim_slice)
+static inline MarchWs march_ws_layout(int64_t n)
 {
     MarchWs L;
-    L.spill_cap = max_prim_slice > RGX_LDS_HITS ? max_prim_slice - RGX_LDS_HITS : 0;
-    size_t off = 0;
-    L.gbuf = off;  off = rgx_align_up(off + (size_t)(n > 0 ? n : 1) * 16 * sizeof(float), 256);
-    L.spill = off; off = rgx_align_up(off + (size_t)(n_rays > 0 ? n_rays : 1) * (size_t)L.spill_cap * sizeof(int32_t), 256);
-    L.total = off;
+    L.gbuf = 0;
+    L.total = rgx_align_up((size_t)(n > 0 ? n : 1) * 16 * sizeof(float), 256);
     return L;
 }
 
 extern "C" int rgx_march_workspace_bytes(int64_t n, int64_t n_rays, int32_t max_prim_slice, size_t *bytes)
 {
     if (n < 0 || n_rays < 0 || max_prim_slice < 0 || !bytes) return RGX_EINVAL;
-    *bytes = march_ws_layout(n, n_rays, max_prim_slice).total;
+    *bytes = march_ws_layout(n).total;
     return RGX_OK;
 }
 
@@ -549,14 +911,14 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     if (!ws || !cam || !march || n < 0 || (n > 0 && !prims) || cam->width <= 0 || cam->height <= 0 ||
         march->max_prim_slice < 0 || !(march->dt_step > 0.0f) || ((uintptr_t)prims & 15u))
         return RGX_EINVAL;
-    const int64_t n_rays = (int64_t)cam->width * cam->height;
-    const MarchWs M = march_ws_layout(n, n_rays, march->max_prim_slice);
+    const MarchWs M = march_ws_layout(n);
     if (!march_ws || march_ws_bytes < M.total || ((uintptr_t)march_ws & 255u)) return RGX_EWORKSPACE;
     const WsLayout L = rgx_ws_layout(n);
     const char *w = (const char *)ws;
     P.cam = *cam;
     P.m = *march;
     P.nodes = (const Node *)(w + L.nodes);
+    P.right = (const int32_t *)(w + L.right);
     P.order = (const uint32_t *)(w + L.vals0);
     P.hdr = (const WsHeader *)(w + L.header);
     P.prims = (const Prim *)prims;
@@ -565,8 +927,6 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     P.fwd_colors = nullptr;
     P.dloss = nullptr;
     P.gbuf = (float *)((char *)march_ws + M.gbuf);
-    P.spill = M.spill_cap ? (int32_t *)((char *)march_ws + M.spill) : nullptr;
-    P.spill_cap = M.spill_cap;
     P.stats = stats;
     P.tiles_x = (cam->width + 7) / 8;
     P.tiles_y = (cam->height + 7) / 8;
@@ -626,6 +986,7 @@ static int hook_params(MarchParams &P, const void *ws, const float *prims, int64
     const char *w = (const char *)ws;
     P = MarchParams{};
     P.nodes = (const Node *)(w + L.nodes);
+    P.right = (const int32_t *)(w + L.right);
     P.order = (const uint32_t *)(w + L.vals0);
     P.hdr = (const WsHeader *)(w + L.header);
     P.prims = (const Prim *)prims;
@@ -658,6 +1019,21 @@ extern "C" int rgx_trace_segments(const void *ws, const float *prims, int64_t n_
     if (n == 0) return RGX_OK;
     hipLaunchKernelGGL(k_trace_segments, grid_for(n, 64), dim3(64), 0, (hipStream_t)stream, P, f3{eye[0], eye[1], eye[2]}, n,
                        dirs, tlo, thi, (int)cap, counts, ids);
+    RGX_LAUNCH_CHECK();
+    return RGX_OK;
+}
+
+extern "C" int rgx_collect_tiles(const void *ws, const RgxCamera *cam, const float *prims, int64_t n_prims, const float *tlo,
+                                 const float *thi, int32_t cap, int32_t *counts, int32_t *ids, void *stream)
+{
+    MarchParams P;
+    const int rc = hook_params(P, ws, prims, n_prims);
+    if (rc) return rc;
+    if (!cam || cam->width <= 0 || cam->height <= 0 || cap <= 0 || !tlo || !thi || !counts || !ids) return RGX_EINVAL;
+    P.cam = *cam;
+    P.tiles_x = (cam->width + 7) / 8;
+    P.tiles_y = (cam->height + 7) / 8;
+    hipLaunchKernelGGL(k_collect_tiles, march_grid(P), dim3(64), 0, (hipStream_t)stream, P, tlo, thi, (int)cap, counts, ids);
     RGX_LAUNCH_CHECK();
     return RGX_OK;
 }

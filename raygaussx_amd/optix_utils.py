@@ -281,3 +281,13 @@ def trace_segments(gas, prims, eye, dirs, tlo, thi, cap):
                                        C.c_int64(n), L.ptr(dirs), L.ptr(tlo), L.ptr(thi), C.c_int32(cap),
                                        L.ptr(counts), L.ptr(ids), L.stream(dirs.device)))
     return counts, ids
+
+
+def collect_tiles(gas, cam, prims, tlo, thi, cap):
+    """Hit lists of per-pixel segments through the tile-cooperative collect (test hook)."""
+    n_rays = cam.width * cam.height
+    counts = torch.zeros(n_rays, dtype=torch.int32, device=prims.device)
+    ids = torch.full((n_rays, cap), -1, dtype=torch.int32, device=prims.device)
+    L.check(L.lib().rgx_collect_tiles(L.ptr(gas.ws), C.byref(cam), L.ptr(prims), C.c_int64(prims.shape[0]), L.ptr(tlo),
+                                      L.ptr(thi), C.c_int32(cap), L.ptr(counts), L.ptr(ids), L.stream(prims.device)))
+    return counts, ids

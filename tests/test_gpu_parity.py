@@ -178,6 +178,44 @@ def test_forward_config0_image_and_hit_sets(gx, orc, c0):
         assert sorted(ids[s, :cnt[s]].tolist()) == want[s], s
 
 
+def test_tile_cooperative_collect_hit_sets_bit_exact(gx, orc, c0):
+    """The collect query as the march kernels run it (one 8x8 tile per wavefront, shared candidate
+    gather, per-ray exact predicate) on the oracle's own slab intervals: identical hit sets."""
+    from raygaussx_amd import optix_utils as u_ox
+    sc, cam, cfg = c0
+    img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"])
+    d = gx.to_dev(sc)
+    gas = u_ox.AccelerationStructure(4096, gx.DEV).build_from_gaussians(d["positions"], d["scales"], d["quaternions"],
+                                                                         d["densities"])
+    ps = u_ox.pack_prims(gas, ctx["eye"], d["positions"], d["scales"], d["quaternions"], d["densities"],
+                         torch.from_numpy(ctx["rgb"]).to(gx.DEV))
+    R = 128 * 128
+    traces = [orc.march_trace(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], r)[0] for r in range(R)]
+    cams = u_ox.camera_struct(cam)
+    checked = 0
+    for rank in (0, 1, 4, 9):
+        tlo = np.ones(R, np.float32)
+        thi = np.zeros(R, np.float32)          # thi < tlo: pixel idle
+        for r in range(R):
+            if len(traces[r]) > rank:
+                tlo[r], thi[r] = traces[r][rank][2], traces[r][rank][3]
+        _step(f"collect_tiles slab rank {rank}")
+        cnt, ids = u_ox.collect_tiles(gas, cams, ps, torch.from_numpy(tlo).to(gx.DEV), torch.from_numpy(thi).to(gx.DEV), 64)
+        cnt, ids = cnt.cpu().numpy(), ids.cpu().numpy()
+        for r in range(R):
+            want = sorted(traces[r][rank][4].tolist()) if len(traces[r]) > rank else []
+            assert sorted(ids[r, :cnt[r]].tolist()) == want, (rank, r)
+            checked += len(want)
+    assert checked > 20000
+    # the max_prim_slice cut is reported per ray
+    tlo = np.full(R, 3.0, np.float32)
+    thi = np.full(R, 5.0, np.float32)
+    cnt, _ = u_ox.collect_tiles(gas, cams, ps, torch.from_numpy(tlo).to(gx.DEV), torch.from_numpy(thi).to(gx.DEV), 3)
+    dirs = orc.ray_dirs(ctx["cs"])
+    c_cpu, _ = orc.trace_segments(ctx["prims"], dirs, tlo, thi, 3)
+    np.testing.assert_array_equal(cnt.cpu().numpy(), c_cpu)
+
+
 def _check_grads(gx, got, want, keys=("positions", "scales", "quaternions", "densities", "color_features")):
     for k in keys:
         cos, rel = gx.cos_rel(got[k], want[k])

@@ -66,6 +66,8 @@ typedef struct RgxStats {
     unsigned long long overflow_rays; /* collect queries truncated at max_prim_slice */
     unsigned long long rays_hit;      /* rays whose first-hit query found a Gaussian */
     unsigned long long nodes_visited; /* BVH nodes fetched by all queries */
+    unsigned long long candidates;     /* Gaussians gathered per tile and slab iteration (filter passes) */
+    unsigned long long candidates_hit; /* ... of which at least one ray of the tile hit */
 } RgxStats;
 
 int rgx_abi_version(void);

@@ -9,7 +9,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "librgx.so")
+# RGX_LIB_PATH selects another build of the same library (e.g. one compiled with extra flags)
+LIB_PATH = os.environ.get("RGX_LIB_PATH") or os.path.join(_HERE, "librgx.so")
 
 
 class RgxError(RuntimeError):
@@ -27,7 +28,8 @@ class RgxMarch(C.Structure):
                 ("white_background", C.c_int32), ("t_eps", C.c_float)]
 
 
-STATS_FIELDS = ("hit_pairs", "slabs", "empty_slabs", "overflow_rays", "rays_hit", "nodes_visited")
+STATS_FIELDS = ("hit_pairs", "slabs", "empty_slabs", "overflow_rays", "rays_hit", "nodes_visited", "candidates",
+                "candidates_hit")
 
 # every symbol include/rgx.h declares
 SYMBOLS = ("rgx_abi_version", "rgx_strerror", "rgx_last_hip_error", "rgx_aabb", "rgx_sh_forward",

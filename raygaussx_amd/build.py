@@ -19,11 +19,12 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-Wno-unused-command-line-argument"]
 
 
-def build(verbose=False, extra=()):
+def build(verbose=False, extra=(), lib=LIB, tag=""):
+    """``extra``: more hipcc flags; ``lib`` / ``tag``: write a differently named library and objects."""
     objs = []
     procs = []
     for src in SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        obj = os.path.join(CSRC, src.replace(".hip", tag + ".o"))
         cmd = ["hipcc", *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
@@ -40,9 +41,9 @@ def build(verbose=False, extra=()):
             print(out)
     if failed:
         raise RuntimeError("hipcc failed")
-    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]
+    cmd = ["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", lib]
     subprocess.check_call(cmd)
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":

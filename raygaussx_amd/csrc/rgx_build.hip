@@ -166,33 +166,51 @@ __global__ __launch_bounds__(RGX_RS_THREADS) void k_rs_hist(const K *__restrict_
     hist[(size_t)threadIdx.x * nblocks + blockIdx.x] = h[threadIdx.x];
 }
 
-__global__ __launch_bounds__(1024) void k_rs_scan(uint32_t *__restrict__ hist, int64_t total)
+// Exclusive scan of the (digit, tile) counts in two levels: block d scans its digit's row of tile
+// counts in place and leaves the row total; one more block scans the 256 totals into digit bases.
+__global__ __launch_bounds__(256) void k_rs_scan_rows(uint32_t *__restrict__ hist, int nblocks, uint32_t *__restrict__ totals)
 {
-    __shared__ uint32_t part[1024];
-    const int64_t per = (total + 1023) / 1024;
-    const int64_t b = threadIdx.x * per, e = b + per < total ? b + per : total;
-    uint32_t s = 0;
-    for (int64_t i = b; i < e; ++i) s += hist[i];
-    part[threadIdx.x] = s;
+    __shared__ uint32_t part[256];
+    uint32_t *row = hist + (size_t)blockIdx.x * nblocks;
+    uint32_t carry = 0;
+    for (int base = 0; base < nblocks; base += 256) {
+        const int i = base + threadIdx.x;
+        const uint32_t v = i < nblocks ? row[i] : 0u;
+        part[threadIdx.x] = v;
+        __syncthreads();
+        for (int o = 1; o < 256; o <<= 1) { // Hillis-Steele inclusive scan
+            const uint32_t t = threadIdx.x >= o ? part[threadIdx.x - o] : 0u;
+            __syncthreads();
+            part[threadIdx.x] += t;
+            __syncthreads();
+        }
+        if (i < nblocks) row[i] = carry + part[threadIdx.x] - v;
+        carry += part[255];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) totals[blockIdx.x] = carry;
+}
+
+__global__ __launch_bounds__(256) void k_rs_scan_totals(uint32_t *__restrict__ totals)
+{
+    __shared__ uint32_t part[256];
+    const uint32_t v = totals[threadIdx.x];
+    part[threadIdx.x] = v;
     __syncthreads();
-    for (int o = 1; o < 1024; o <<= 1) { // Hillis-Steele inclusive scan
-        uint32_t v = threadIdx.x >= o ? part[threadIdx.x - o] : 0;
+    for (int o = 1; o < 256; o <<= 1) {
+        const uint32_t t = threadIdx.x >= o ? part[threadIdx.x - o] : 0u;
         __syncthreads();
-        part[threadIdx.x] += v;
+        part[threadIdx.x] += t;
         __syncthreads();
     }
-    uint32_t run = threadIdx.x ? part[threadIdx.x - 1] : 0;
-    for (int64_t i = b; i < e; ++i) {
-        const uint32_t v = hist[i];
-        hist[i] = run;
-        run += v;
-    }
+    totals[threadIdx.x] = part[threadIdx.x] - v;
 }
 
 template <typename K>
 __global__ __launch_bounds__(RGX_RS_THREADS) void k_rs_scatter(const K *__restrict__ kin, const uint32_t *__restrict__ vin,
                                                                K *__restrict__ kout, uint32_t *__restrict__ vout, int64_t n,
-                                                               int shift, const uint32_t *__restrict__ hist, int nblocks)
+                                                               int shift, const uint32_t *__restrict__ hist, int nblocks,
+                                                               const uint32_t *__restrict__ digit_base)
 {
     __shared__ uint32_t cnt[4][256];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -215,7 +233,7 @@ __global__ __launch_bounds__(RGX_RS_THREADS) void k_rs_scatter(const K *__restri
     __syncthreads();
     {
         const int d = threadIdx.x;
-        uint32_t run = hist[(size_t)d * nblocks + blockIdx.x];
+        uint32_t run = digit_base[d] + hist[(size_t)d * nblocks + blockIdx.x];
         for (int w = 0; w < 4; ++w) {
             const uint32_t c = cnt[w][d];
             cnt[w][d] = run;
@@ -254,8 +272,11 @@ static int radix_sort(K *k0, uint32_t *v0, K *k1, uint32_t *v1, int64_t n, int b
     uint32_t *vi = v0, *vo = v1;
     for (int shift = 0; shift < bits; shift += 8) {
         hipLaunchKernelGGL(k_rs_hist<K>, dim3(nblocks), dim3(RGX_RS_THREADS), 0, s, ki, n, shift, hist, nblocks);
-        hipLaunchKernelGGL(k_rs_scan, dim3(1), dim3(1024), 0, s, hist, (int64_t)256 * nblocks);
-        hipLaunchKernelGGL(k_rs_scatter<K>, dim3(nblocks), dim3(RGX_RS_THREADS), 0, s, ki, vi, ko, vo, n, shift, hist, nblocks);
+        uint32_t *totals = hist + (size_t)256 * nblocks;
+        hipLaunchKernelGGL(k_rs_scan_rows, dim3(256), dim3(256), 0, s, hist, nblocks, totals);
+        hipLaunchKernelGGL(k_rs_scan_totals, dim3(1), dim3(256), 0, s, totals);
+        hipLaunchKernelGGL(k_rs_scatter<K>, dim3(nblocks), dim3(RGX_RS_THREADS), 0, s, ki, vi, ko, vo, n, shift, hist, nblocks,
+                           totals);
         K *tk = ki; ki = ko; ko = tk;
         uint32_t *tv = vi; vi = vo; vo = tv;
     }
@@ -318,6 +339,19 @@ __global__ __launch_bounds__(256) void k_karras(const uint64_t *__restrict__ key
     parent[rc] = (int32_t)i;
 }
 
+// Bottom-up refit: every leaf walks towards the root; the second thread to reach a node
+// (counted with an atomic) merges the two child boxes and goes on.  Box words travel between
+// threads through agent-scope atomic stores and loads (coherent across the XCDs' L2s without a
+// cache write-back); the workgroup-scope fences only order them against the counter.
+__device__ __forceinline__ void st_agent(float *p, float v)
+{
+    __hip_atomic_store((int *)p, __float_as_int(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float ld_agent(const float *p)
+{
+    return __int_as_float(__hip_atomic_load((const int *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+
 __global__ __launch_bounds__(256) void k_refit(int64_t n, Node *nodes, const int32_t *__restrict__ parent,
                                                const int32_t *__restrict__ right, int32_t *flags)
 {
@@ -325,16 +359,14 @@ __global__ __launch_bounds__(256) void k_refit(int64_t n, Node *nodes, const int
     if (j >= n) return;
     int32_t node = parent[n - 1 + j];
     while (node >= 0) {
-        __threadfence();
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (atomicAdd(&flags[node], 1) == 0) return; // the sibling subtree is not done yet
-        __threadfence();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
         const Node *a = &nodes[nodes[node].left];
         const Node *b = &nodes[right[node]];
-        // volatile reads: the children were written by other workgroups during this launch
-        const volatile float *al = a->lo, *ah = a->hi, *bl = b->lo, *bh = b->hi;
         for (int c = 0; c < 3; ++c) {
-            nodes[node].lo[c] = fminf(al[c], bl[c]);
-            nodes[node].hi[c] = fmaxf(ah[c], bh[c]);
+            st_agent(&nodes[node].lo[c], fminf(ld_agent(&a->lo[c]), ld_agent(&b->lo[c])));
+            st_agent(&nodes[node].hi[c], fmaxf(ld_agent(&a->hi[c]), ld_agent(&b->hi[c])));
         }
         node = parent[node];
     }
@@ -551,7 +583,7 @@ static inline MortonLayout morton_layout(int64_t n)
     L.keys1 = off; off = rgx_align_up(off + nn * 4, 256);
     L.vals0 = off; off = rgx_align_up(off + nn * 4, 256);
     L.vals1 = off; off = rgx_align_up(off + nn * 4, 256);
-    L.hist = off;  off = rgx_align_up(off + 256 * nblocks * 4, 256);
+    L.hist = off;  off = rgx_align_up(off + 256 * (nblocks + 1) * 4, 256);
     L.total = off;
     return L;
 }

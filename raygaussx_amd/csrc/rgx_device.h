@@ -143,7 +143,7 @@ static inline WsLayout rgx_ws_layout(int64_t n)
     L.parent = off; off = rgx_align_up(off + (2 * nn) * sizeof(int32_t), 256);
     L.right = off;  off = rgx_align_up(off + nn * sizeof(int32_t), 256);
     L.flags = off;  off = rgx_align_up(off + nn * sizeof(int32_t), 256);
-    L.hist = off;   off = rgx_align_up(off + 256 * nblocks * sizeof(uint32_t), 256);
+    L.hist = off;   off = rgx_align_up(off + 256 * (nblocks + 1) * sizeof(uint32_t), 256);
     L.total = off;
     return L;
 }

@@ -43,6 +43,7 @@ struct MarchParams {
 struct Counters {
     unsigned hit_pairs = 0, slabs = 0, empty = 0, overflow = 0, rays_hit = 0;
     unsigned long long nodes = 0;
+    unsigned cands = 0, cands_hit = 0; // per wave (lane 0 counts)
 };
 
 // ---------------------------------------------------------------------------
@@ -314,8 +315,8 @@ __device__ __forceinline__ bool tile_origin(const MarchParams &P, int &px0, int 
 __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
 {
     if (!st) return;
-    unsigned long long v[6] = {c.hit_pairs, c.slabs, c.empty, c.overflow, c.rays_hit, c.nodes};
-    for (int k = 0; k < 6; ++k) {
+    unsigned long long v[8] = {c.hit_pairs, c.slabs, c.empty, c.overflow, c.rays_hit, c.nodes, c.cands, c.cands_hit};
+    for (int k = 0; k < 8; ++k) {
         unsigned long long x = v[k];
         for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
         v[k] = x;
@@ -323,6 +324,7 @@ __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
     if ((threadIdx.x & 63) == 0) {
         atomicAdd(&st->hit_pairs, v[0]); atomicAdd(&st->slabs, v[1]); atomicAdd(&st->empty_slabs, v[2]);
         atomicAdd(&st->overflow_rays, v[3]); atomicAdd(&st->rays_hit, v[4]); atomicAdd(&st->nodes_visited, v[5]);
+        atomicAdd(&st->candidates, v[6]); atomicAdd(&st->candidates_hit, v[7]);
     }
 }
 
@@ -453,10 +455,16 @@ __device__ __forceinline__ void pass_filter(const MarchParams &P, const Frustum 
         }
         first = false;
         uint32_t mask = 0;
+#ifdef RGX_EXP_NOFILTER
+        if (C >= 0) { p0 = 1; continue; }
+#endif
         for (int c = 0; c < C; ++c) {
             const int pid = __builtin_amdgcn_readfirstlane(s_cand[c]);
             const Prim p = P.prims[pid];
             const bool hit = lane_hits(p, dir, run, tlo, thi, cap, p0, ov);
+#ifdef RGX_EXP_NOSHADE
+            continue;
+#endif
             if (rec) {
                 mask |= (uint32_t)hit << (c & 31);
                 if ((c & 31) == 31 || c == C - 1) {
@@ -464,8 +472,12 @@ __device__ __forceinline__ void pass_filter(const MarchParams &P, const Frustum 
                     mask = 0;
                 }
             }
-            if (__ballot(hit)) body(p, pid, hit);
+            if (__ballot(hit)) {
+                if (lane == 0) cn.cands_hit++;
+                body(p, pid, hit);
+            }
         }
+        if (lane == 0) cn.cands += (unsigned)C;
     } while (!done);
 }
 

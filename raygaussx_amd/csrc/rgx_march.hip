@@ -12,14 +12,15 @@
 //      predicate for ITS ray and slab (so hit sets are those of a per-ray query),
 //      and the lanes that hit accumulate the candidate's samples.  Candidate data
 //      is wave-uniform, i.e. one 64-byte fetch per wave instead of one per lane;
-//   3. (backward) reduces each candidate's 14 gradient words across the wave with
-//      DPP adds and issues ONE set of atomics per wave and candidate.
-// The first-hit query (once per ray, and after an empty slab) walks the BVH per lane
-// through its skip links.
+//   3. (backward) sums each candidate's 14 gradient words over the 16 rays of a 4x4
+//      pixel row with DPP adds and issues ONE set of atomics per row and candidate.
+// The first-hit query (once per ray, and after an empty slab) runs on the same
+// candidate tables.  The per-lane skip-link queries below serve the segment test
+// hooks (arbitrary rays).
 #include "rgx_device.h"
 
-#define RGX_QCAP 2048      // node stack entries per wave (LDS)
-#define RGX_CCAP 256       // candidate table entries per wave (LDS)
+#define RGX_QCAP 1024      // node stack entries per wave (LDS)
+#define RGX_CCAP 128       // candidate table entries per wave (LDS)
 #define RGX_DFS_MARGIN 192 // above QCAP - margin the sweep pops one node at a time (depth-first)
 #define RGX_LDS_HITS 32    // per-lane list of the stand-alone collect hook
 
@@ -216,11 +217,23 @@ __device__ __forceinline__ bool frustum_overlaps(const Frustum &F, float4 a, flo
     return !out;
 }
 
-// Cooperative sweep of the BVH: the node stack is shared by the wave, every step pops
-// up to 64 nodes (one per lane), tests them against the frustum, appends the leaves
-// that pass to the candidate table and pushes the children of the internal nodes that
-// pass.  Returns when the stack is empty (done) or the table might not take another
-// step's leaves; call again to continue with an emptied table.
+// Candidate table.  A Gaussian that survives the sweep is turned, by the lane that found
+// it, into everything the per-ray work needs and parked in LDS, where all lanes later read
+// it as a broadcast: rotation columns, the ray-independent half of the hit predicate
+// (S^-1 R^T (eye - centre) and its squared norm - 1), and the distance shell [dmin, dmax]
+// from the eye that bounds the ellipsoid.  The values are produced by the same operations,
+// in the same order, as in line_roots(), so using them changes no rounding.
+//   float4 0: U.xyz, dmin     1: V.xyz, dmax     2: W.xyz, k      3: inv_inter.xyz, c
+//          4: Oe.xyz, rho     5: (eye-centre).xyz, sorted index   6: rgb*rho, -
+#define RGX_TAB 28
+
+// Cooperative sweep of the BVH: the node stack is shared by the wave, every step pops up to
+// 64 nodes (one per lane) and tests their boxes against the frustum.  Internal nodes that pass
+// push their children.  A leaf that passes is tested again with its actual ellipsoid -- exact
+// support distance against the four frustum planes, bounding sphere against the shell -- and,
+// if it still passes, written to the candidate table.  Returns the number of table entries
+// when the stack is empty (done) or the table might not take another step's leaves; call again
+// to continue with an emptied table.
 struct Sweep {
     int qn; // stack entries (wave-uniform)
 };
@@ -232,7 +245,7 @@ __device__ __forceinline__ void sweep_begin(const MarchParams &P, Sweep &S, int3
     __syncthreads();
 }
 
-__device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int32_t *s_queue, int32_t *s_cand, bool &done,
+__device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int32_t *s_queue, float *s_tab, bool &done,
                           Counters &cn)
 {
     const int lane = threadIdx.x;
@@ -259,8 +272,46 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
             }
         }
         if (lane == 0) cn.nodes += (unsigned)m;
+        float4 e[7];
+        if (leaf_hit) {
+            const int32_t pid = ~left;
+            const Prim p = P.prims[pid];
+            f3 U, V, W;
+            quat_to_cols(p.quat4, U, V, W);
+            const f3 inv = mk3(p.inv_inter4.x, p.inv_inter4.y, p.inv_inter4.z);
+            const f3 O = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
+            // semi-axes of the k-sigma ellipsoid: k * scale = 1 / inv_inter
+            const f3 ax = mk3(1.0f / inv.x, 1.0f / inv.y, 1.0f / inv.z);
+            const float dist = sqrtf(dot3(O, O));
+            const float rad = fmaxf(ax.x, fmaxf(ax.y, ax.z)) * 1.001f + 1e-5f * dist + F.pad;
+            const float dmin = dist - rad, dmax = dist + rad;
+            bool ok = p.inv_inter4.w == p.inv_inter4.w; // k is NaN below the density threshold: never hit
+            ok = ok && dmax >= F.t0 && dmin <= F.t1;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const f3 n = F.n[k];
+                // the ellipsoid reaches h beyond its centre along n; centre - eye = -O
+                const float hu = dot3(U, n) * ax.x, hv = dot3(V, n) * ax.y, hw = dot3(W, n) * ax.z;
+                const float h = sqrtf((hu * hu + hv * hv) + hw * hw) * 1.001f;
+                ok = ok && !(-dot3(n, O) - h > F.pad);
+            }
+            leaf_hit = ok;
+            const f3 Oe = apply_sinv_rt(O, U, V, W, inv);
+            const float cc = fmaf(Oe.x, Oe.x, fmaf(Oe.y, Oe.y, fmaf(Oe.z, Oe.z, -1.0f)));
+            e[0] = make_float4(U.x, U.y, U.z, dmin);
+            e[1] = make_float4(V.x, V.y, V.z, dmax);
+            e[2] = make_float4(W.x, W.y, W.z, p.inv_inter4.w);
+            e[3] = make_float4(inv.x, inv.y, inv.z, cc);
+            e[4] = make_float4(Oe.x, Oe.y, Oe.z, p.rgba4.w);
+            e[5] = make_float4(O.x, O.y, O.z, __int_as_float(pid));
+            e[6] = make_float4(p.rgba4.x, p.rgba4.y, p.rgba4.z, 0.f);
+        }
         const uint64_t bl = __ballot(leaf_hit), bi = __ballot(inner_hit);
-        if (leaf_hit) s_cand[C + __popcll(bl & lt)] = ~left;
+        if (leaf_hit) {
+            float4 *dst = (float4 *)(s_tab + (C + __popcll(bl & lt)) * RGX_TAB);
+#pragma unroll
+            for (int k = 0; k < 7; ++k) dst[k] = e[k];
+        }
         C += __popcll(bl);
         if (inner_hit) {
             const int pos = S.qn + 2 * __popcll(bi & lt);
@@ -275,29 +326,6 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
     }
     done = S.qn == 0;
     return C;
-}
-
-// Per-hit constants of the sample recurrence (gaussians_aabb.cu:135-164).
-struct HitSetup {
-    float power, inc, inc_st, cut;
-};
-__device__ __forceinline__ HitSetup hit_setup(const Prim &p, f3 dir, f3 ray_dir_tmid, float dt)
-{
-    const float k = p.inv_inter4.w;
-    const f3 inv_s = mk3(p.inv_inter4.x * k, p.inv_inter4.y * k, p.inv_inter4.z * k);
-    f3 U, V, W;
-    quat_to_cols(p.quat4, U, V, W);
-    const f3 xhit = mk3(p.pos4.x, p.pos4.y, p.pos4.z) + ray_dir_tmid;
-    const f3 Mx0 = apply_sinv_rt(xhit, U, V, W, inv_s);
-    const f3 Md = apply_sinv_rt(dir, U, V, W, inv_s);
-    const float Md2 = dot3(Md, Md);
-    const float Md_dt_2 = (dt * dt) * Md2;
-    HitSetup h;
-    h.power = dot3(Mx0, Mx0);
-    h.inc = Md_dt_2 + 2.0f * dot3(Mx0, Md) * dt;
-    h.inc_st = 2.0f * Md_dt_2;
-    h.cut = k * k;
-    return h;
 }
 
 __device__ __forceinline__ bool tile_origin(const MarchParams &P, int &px0, int &py0)
@@ -329,17 +357,24 @@ __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
 }
 
 // State of one ray between slab iterations; the slab loop itself is wave-uniform.
+// A ray is either marching (its next slab is [tbuffer, tbuffer + 32 dt]) or searching:
+// looking for the first Gaussian at or after tbuffer -- the reference's first-hit query
+// (optixTrace SBT offset 0), issued once per ray (gaussians_aabb.cu:234-257) and after
+// every empty slab (297-319).  The search runs on the same candidate tables as the slabs,
+// one window per iteration: if no Gaussian of the window is hit at or after tbuffer, every
+// hit lies beyond the window, so searching on from the window's end returns the same
+// closest t as one query over [tbuffer, texit] would.
 struct RayState {
     f3 dir;
     float tenter, texit, tbuffer, T, dt, slab_spacing;
-    bool active;
+    bool active, searching, first;
 };
 
-// Ray set-up up to the first hit: computeRay, scene-bbox slab test, first-hit query
-// (fwd: gaussians_aabb.cu:207-260; bwd: backward/gaussians_aabb.cu:211-254, which divides
-// by the direction where the forward multiplies by its reciprocal).
+// Ray set-up: computeRay and the scene-bbox slab test (fwd: gaussians_aabb.cu:207-231;
+// bwd: backward/gaussians_aabb.cu:211-233, which divides by the direction where the forward
+// multiplies by its reciprocal).  The ray starts out searching from the box entry.
 template <bool DIVIDE>
-__device__ __forceinline__ void ray_begin(const MarchParams &P, int px, int py, bool valid, RayState &R, Counters &cn)
+__device__ __forceinline__ void ray_begin(const MarchParams &P, int px, int py, bool valid, RayState &R)
 {
     const f3 o = mk3(P.cam.eye[0], P.cam.eye[1], P.cam.eye[2]);
     R.dir = compute_ray(P.cam, (unsigned)px, (unsigned)py);
@@ -360,20 +395,17 @@ __device__ __forceinline__ void ray_begin(const MarchParams &P, int px, int py, 
     R.dt = P.m.dt_step;
     R.slab_spacing = R.dt * RGX_BUFFER_SIZE;
     R.T = 1.0f;
-    R.active = false;
-    R.tbuffer = 0.f;
-    if (valid) {
-        const float fh = first_hit(P, o, R.dir, R.tenter, R.texit, cn);
-        if (fh != -1.0f) {
-            cn.rays_hit++;
-            R.tenter = fh;
-            R.active = R.tenter < R.texit;
-            R.tbuffer = R.tenter;
-        }
-    }
+    R.tbuffer = R.tenter;
+    R.searching = true;
+    R.first = true;
+    // a first hit can only be reported inside [tenter, texit]; with tenter >= texit the ray keeps
+    // the background either way (gaussians_aabb.cu:249-260, 333-339)
+    R.active = valid && P.n > 0 && R.tenter < R.texit;
 }
 
-// Top of a slab iteration: loop condition, adaptive step (gaussians_aabb.cu:266-276), slab bounds.
+// Top of an iteration: loop condition, adaptive step (gaussians_aabb.cu:266-276) and the interval
+// this ray asks about: its slab when marching (returns true), or one slab length ahead of tbuffer
+// when searching (returns false; the search itself runs to the end of the candidate window).
 // CLIP: the forward clips the slab to [tenter, texit] (275-276), the backward does not (279-280).
 template <bool CLIP>
 __device__ __forceinline__ bool slab_begin(const MarchParams &P, RayState &R, float &tlo, float &thi)
@@ -381,128 +413,276 @@ __device__ __forceinline__ bool slab_begin(const MarchParams &P, RayState &R, fl
     R.active = R.active && R.tbuffer < R.texit && R.T > P.m.t_eps;
     // a step below one ulp of t cannot advance the ray: stop instead of spinning
     R.active = R.active && (R.tbuffer + R.slab_spacing > R.tbuffer);
-    if (R.active && P.m.dynamic_sampling) {
+    if (R.active && !R.searching && P.m.dynamic_sampling) {
         const float dt_dist = fmaxf(R.tbuffer / 1024.0f, P.m.dt_step);
         const float coeff = rcbrtf(R.T);
         R.dt = fminf(dt_dist * coeff, 4.0f * P.m.dt_step);
         R.slab_spacing = R.dt * RGX_BUFFER_SIZE;
+    }
+    if (R.searching) {
+        tlo = R.tbuffer;
+        thi = fminf(R.texit, R.tbuffer + R.slab_spacing);
+        return false;
     }
     tlo = CLIP ? fmaxf(R.tenter, R.tbuffer) : R.tbuffer;
     thi = CLIP ? fminf(R.texit, R.tbuffer + R.slab_spacing) : R.tbuffer + R.slab_spacing;
     return R.active && thi > R.tenter;
 }
 
-// End of a slab iteration for this ray: skip ahead after an empty slab
-// (gaussians_aabb.cu:297-319) or step to the next slab (324).
-__device__ __forceinline__ void slab_end(const MarchParams &P, RayState &R, bool need, int p0, Counters &cn)
+// End of an iteration.  Marching ray: step to the next slab; after an empty slab start searching
+// from there (gaussians_aabb.cu:297-319, 324).  Searching ray: `found` (< 0: nothing in
+// [tbuffer, searched_to]) either restarts the march at the hit or moves the search on.
+__device__ __forceinline__ void slab_end(RayState &R, bool need, int p0, float found, float searched_to, Counters &cn)
 {
     if (!R.active) return;
+    if (R.searching) {
+        if (found >= 0.0f) {
+            if (R.first) {
+                R.first = false;
+                cn.rays_hit++;
+                R.tenter = found;
+                R.active = found < R.texit;
+            }
+            R.tbuffer = found;
+            R.searching = false;
+        } else {
+            R.tbuffer = searched_to;
+            R.active = searched_to < R.texit;
+        }
+        return;
+    }
+    R.tbuffer += R.slab_spacing;
     if (need && p0 == 0) {
         cn.empty++;
-        R.tbuffer += R.slab_spacing;
-        const float nt = first_hit(P, mk3(P.cam.eye[0], P.cam.eye[1], P.cam.eye[2]), R.dir, R.tbuffer, R.texit, cn);
-        if (nt == -1.0f) R.active = false;
-        else R.tbuffer = nt;
-    } else {
-        R.tbuffer += R.slab_spacing;
+        R.searching = true;
     }
-}
-
-// Exact per-ray hit test of one candidate (the collect query's __intersection__gaussian +
-// __anyhit__ah, gaussians_aabb.cu:36-92, 349-367) with the max_prim_slice cut.
-__device__ __forceinline__ bool lane_hits(const Prim &p, f3 dir, bool need, float tlo, float thi, int cap, int &p0, bool &ov)
-{
-    if (!need || ov) return false;
-    float r1, r2, t;
-    if (!(line_roots(p.pos4, p.inv_inter4, p.quat4, dir, r1, r2) && segment_hit(r1, r2, tlo, thi, t))) return false;
-    if (p0 >= cap) {
-        ov = true; // optixTerminateRay: this ray collects nothing further in this slab
-        return false;
-    }
-    ++p0;
-    return true;
 }
 
 // ---------------------------------------------------------------------------
-// One pass over all candidates of the current slab iteration.
-//
-// pass_filter sweeps the BVH (in as many table-fuls as needed), evaluates the exact
-// predicate per lane and calls body(prim, pid, hit) for every candidate some lane
-// hits.  When the whole candidate set fitted in ONE table it also records each lane's
-// hit bits, so that a later pass over the same slab (second chunk, gradient pass) can
-// replay them with pass_replay instead of sweeping and testing again.
-struct PassState {
-    int n_saved;   // candidates held in the table (valid when single)
-    bool single;   // the last filter pass needed one table only
+struct TileLds {
+    int32_t *queue;        // [RGX_QCAP]
+    float *tab;            // [RGX_CCAP * RGX_TAB]
+    uint8_t *rowlist;      // [4][RGX_CCAP]: per 16-lane row, table slots some lane of the row hits
+    uint32_t (*mask)[64];  // [RGX_CCAP / 32][64]: per lane, hit bits over its row's list
 };
 
-template <typename Body>
-__device__ __forceinline__ void pass_filter(const MarchParams &P, const Frustum &F, int32_t *s_queue, int32_t *s_cand,
-                                            uint32_t (*s_mask)[64], PassState &ps, bool record, f3 dir, bool run, float tlo,
-                                            float thi, int cap, int &p0, bool &ov, Counters &cn, Body body)
+// Ray-interval-independent half of __intersection__gaussian (gaussians_aabb.cu:43-82) on a table
+// entry: same arithmetic as line_roots(), with the precomputed ray-independent parts.
+__device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, float &r2)
 {
-    const int lane = threadIdx.x;
-    Sweep S;
-    sweep_begin(P, S, s_queue);
-    bool done = false, first = true;
-    ps.single = false;
-    do {
-        const int C = sweep_next(P, S, F, s_queue, s_cand, done, cn);
-        const bool rec = record && first && done;
-        if (first && done) {
-            ps.single = true;
-            ps.n_saved = C;
-        }
-        first = false;
-        uint32_t mask = 0;
-#ifdef RGX_EXP_NOFILTER
-        if (C >= 0) { p0 = 1; continue; }
-#endif
-        for (int c = 0; c < C; ++c) {
-            const int pid = __builtin_amdgcn_readfirstlane(s_cand[c]);
-            const Prim p = P.prims[pid];
-            const bool hit = lane_hits(p, dir, run, tlo, thi, cap, p0, ov);
-#ifdef RGX_EXP_NOSHADE
-            continue;
-#endif
-            if (rec) {
-                mask |= (uint32_t)hit << (c & 31);
-                if ((c & 31) == 31 || c == C - 1) {
-                    s_mask[c >> 5][lane] = mask;
-                    mask = 0;
-                }
-            }
-            if (__ballot(hit)) {
-                if (lane == 0) cn.cands_hit++;
-                body(p, pid, hit);
-            }
-        }
-        if (lane == 0) cn.cands += (unsigned)C;
-    } while (!done);
+    const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3], e4 = e[4];
+    const f3 De = apply_sinv_rt(dir, mk3(e0.x, e0.y, e0.z), mk3(e1.x, e1.y, e1.z), mk3(e2.x, e2.y, e2.z), mk3(e3.x, e3.y, e3.z));
+    const f3 Oe = mk3(e4.x, e4.y, e4.z);
+    const float a = fmaf(De.x, De.x, fmaf(De.y, De.y, De.z * De.z));
+    const float b = -fmaf(Oe.x, De.x, fmaf(Oe.y, De.y, Oe.z * De.z));
+    const float c = e3.w;
+    const float inv_a = 1.0f / a;
+    const float b_inv_a = b * inv_a;
+    const f3 Pc = mk3(fmaf(b_inv_a, De.x, Oe.x), fmaf(b_inv_a, De.y, Oe.y), fmaf(b_inv_a, De.z, Oe.z));
+    const float d2 = fmaf(Pc.x, Pc.x, fmaf(Pc.y, Pc.y, Pc.z * Pc.z));
+    const float disc = 1.0f - d2;
+    if (!(disc > 1e-7f)) return false;
+    const float sdisc = sqrtf(disc * a);
+    const float q = b + copysignf(sdisc, b);
+    r1 = c / q;
+    r2 = q * inv_a;
+    return true;
 }
 
-template <typename Body>
-__device__ __forceinline__ void pass_replay(const MarchParams &P, const int32_t *s_cand, uint32_t (*s_mask)[64],
-                                            const PassState &ps, bool run, Body body)
+// Per-hit constants of the sample recurrence (gaussians_aabb.cu:135-164), from a table entry.
+struct HitSetup {
+    float power, inc, inc_st, cut;
+};
+__device__ __forceinline__ HitSetup hit_setup(const float4 *e, f3 dir, f3 ray_dir_tmid, float dt)
 {
-    const int lane = threadIdx.x;
-    uint32_t mask = 0;
-    for (int c = 0; c < ps.n_saved; ++c) {
-        if ((c & 31) == 0) mask = s_mask[c >> 5][lane];
-        const bool hit = run && ((mask >> (c & 31)) & 1u);
+    const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3], e5 = e[5];
+    const float k = e2.w;
+    const f3 inv_s = mk3(e3.x * k, e3.y * k, e3.z * k);
+    const f3 U = mk3(e0.x, e0.y, e0.z), V = mk3(e1.x, e1.y, e1.z), W = mk3(e2.x, e2.y, e2.z);
+    const f3 xhit = mk3(e5.x, e5.y, e5.z) + ray_dir_tmid;
+    const f3 Mx0 = apply_sinv_rt(xhit, U, V, W, inv_s);
+    const f3 Md = apply_sinv_rt(dir, U, V, W, inv_s);
+    const float Md2 = dot3(Md, Md);
+    const float Md_dt_2 = (dt * dt) * Md2;
+    HitSetup h;
+    h.power = dot3(Mx0, Mx0);
+    h.inc = Md_dt_2 + 2.0f * dot3(Mx0, Md) * dt;
+    h.inc_st = 2.0f * Md_dt_2;
+    h.cut = k * k;
+    return h;
+}
+
+// What one lane asks of the candidate table in this iteration.
+struct LaneQuery {
+    f3 dir;
+    bool need;      // marching: collect the hits of [tlo, thi] (the collect query, gaussians_aabb.cu:282-295, 349-367)
+    float tlo, thi;
+    bool search;    // searching: smallest hit t in [slo, shi] (the first-hit query, 234-247, 370-380)
+    float slo, shi;
+    int cap;        // max_prim_slice
+};
+
+// Filter: every lane tests the table entries whose distance shell meets [t0, t1] (the union of
+// the lanes' intervals).  A wave is four 16-lane rows, each row a 4x4 pixel block; an entry hit
+// by any marching lane of a row is appended to that row's list, and each lane keeps its own hit
+// bits over its row's list.  len (row-uniform) is the list length; p0 / ov count this lane's
+// hits and note the max_prim_slice cut (__anyhit__ah's optixTerminateRay, 352-356); found is
+// the running minimum of the searching lanes.
+__device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, float t1, const LaneQuery &Q, int &p0, bool &ov,
+                                             float &found, int &len, Counters &cn)
+{
+    const int lane = threadIdx.x, row = lane >> 4;
+    len = 0;
+    uint32_t bits = 0;
+#ifdef RGX_EXP_NOFILTER
+    if (C >= 0) { p0 = 1; return; }
+#endif
+    for (int h = 0; h < RGX_CCAP / 64; ++h) {
+        const int cl = h * 64 + lane;
+        bool rel = false;
+        if (cl < C) {
+            const float dmin = L.tab[cl * RGX_TAB + 3], dmax = L.tab[cl * RGX_TAB + 7];
+            rel = dmax >= t0 && dmin <= t1;
+        }
+        uint64_t m = __ballot(rel);
+        if (lane == 0) cn.cands += (unsigned)__popcll(m);
+        while (m) {
+            const int c = h * 64 + __builtin_ctzll(m);
+            m &= m - 1;
+            float r1, r2, t;
+            bool hit = false;
+            if ((Q.need && !ov) || Q.search) {
+                if (lane_roots((const float4 *)(L.tab + c * RGX_TAB), Q.dir, r1, r2)) {
+                    if (Q.search) {
+                        if (segment_hit(r1, r2, Q.slo, Q.shi, t)) found = found < 0.0f ? t : fminf(found, t);
+                    } else if (segment_hit(r1, r2, Q.tlo, Q.thi, t)) {
+                        if (p0 >= Q.cap) ov = true;
+                        else {
+                            ++p0;
+                            hit = true;
+                        }
+                    }
+                }
+            }
+            const uint64_t bal = __ballot(hit);
+            if (lane == 0 && bal) cn.cands_hit++;
+            if ((bal >> (row * 16)) & 0xffffull) {
+                bits |= (uint32_t)hit << (len & 31);
+                if ((lane & 15) == 0) L.rowlist[row * RGX_CCAP + len] = (uint8_t)c;
+                ++len;
+                if ((len & 31) == 0) {
+                    L.mask[(len >> 5) - 1][lane] = bits;
+                    bits = 0;
+                }
+            }
+        }
+    }
+    if (len & 31) L.mask[len >> 5][lane] = bits;
+    __syncthreads();
+}
+
+// Shade: the four rows walk their own lists in lock step; body(entry, hit, live) runs whenever
+// some lane hits (hit: this lane hits this entry; live: this lane's row still has an entry at i).
+template <typename Body>
+__device__ __forceinline__ void shade_rows(const TileLds &L, int len, bool run, Body body)
+{
+    const int lane = threadIdx.x, row = lane >> 4;
+    const int l0 = __builtin_amdgcn_readlane(len, 0), l1 = __builtin_amdgcn_readlane(len, 16);
+    const int l2 = __builtin_amdgcn_readlane(len, 32), l3 = __builtin_amdgcn_readlane(len, 48);
+    const int maxlen = max(max(l0, l1), max(l2, l3));
+    uint32_t bits = 0;
+#ifdef RGX_EXP_NOSHADE
+    if (maxlen >= 0) return;
+#endif
+    for (int i = 0; i < maxlen; ++i) {
+        if ((i & 31) == 0) bits = L.mask[i >> 5][lane];
+        const bool live = i < len;
+        const bool hit = run && live && ((bits >> (i & 31)) & 1u);
         if (__ballot(hit)) {
-            const int pid = __builtin_amdgcn_readfirstlane(s_cand[c]);
-            const Prim p = P.prims[pid];
-            body(p, pid, hit);
+            const int c = live ? L.rowlist[row * RGX_CCAP + i] : 0;
+            body((const float4 *)(L.tab + c * RGX_TAB), hit, live);
         }
     }
 }
 
-__device__ __forceinline__ void frustum_range(Frustum &F, bool need, float tlo, float thi)
+// Resident candidate window: the table holds every Gaussian of the tile frustum between the
+// wave's nearest slab start and `hi`, so the next slab iterations reuse it without sweeping.
+struct Window {
+    float hi;
+    int n;
+    bool resident;
+    int k; // slabs to look ahead when a window is built
+};
+
+__device__ __forceinline__ void frustum_range(Frustum &F, float t0, float t1)
 {
-    F.t0 = wave_min_all(need ? tlo : INFINITY);
-    F.t1 = wave_max_all(need ? thi : -INFINITY);
-    F.pad = 2.0f * RGX_PAD_REL * fmaxf(F.t1, 1.0f);
+    F.t0 = t0;
+    F.t1 = t1;
+    F.pad = 2.0f * RGX_PAD_REL * fmaxf(t1, 1.0f);
+}
+
+// Makes the table cover this iteration's slabs.  Returns true when the table is resident
+// (complete); false when even this iteration's own range overflows it, in which case the
+// caller walks the range in table-sized batches.
+__device__ bool window_ensure(const MarchParams &P, const TileLds &L, Frustum &F, Window &Wn, bool need, float tlo,
+                              float slab_spacing, float t0, float t1, Counters &cn)
+{
+    if (Wn.resident && t1 <= Wn.hi) return true;
+    for (;;) {
+        float wend = t1;
+        if (Wn.k > 1) wend = fmaxf(t1, wave_max_all(need ? tlo + (float)Wn.k * slab_spacing : -INFINITY));
+        frustum_range(F, t0, wend);
+        Sweep S;
+        sweep_begin(P, S, L.queue);
+        bool done;
+        const int C = sweep_next(P, S, F, L.queue, L.tab, done, cn);
+        if (done) {
+            Wn.hi = wend;
+            Wn.n = C;
+            Wn.resident = true;
+            if (C > (RGX_CCAP * 3) / 4) Wn.k = Wn.k > 1 ? Wn.k / 2 : 1;
+            else if (C < RGX_CCAP / 3 && Wn.k < 32) Wn.k *= 2;
+            return true;
+        }
+        if (Wn.k == 1) break;
+        Wn.k = 1; // too many Gaussians ahead: retry with this iteration's range only
+    }
+    Wn.resident = false;
+    frustum_range(F, t0, t1);
+    return false;
+}
+
+// Runs `work(C)` on the resident table, or on each table-sized batch of a fresh sweep.
+template <typename Work>
+__device__ __forceinline__ void for_each_table(const MarchParams &P, const TileLds &L, const Frustum &F, const Window &Wn,
+                                               Counters &cn, Work work)
+{
+    if (Wn.resident) {
+        work(Wn.n);
+        return;
+    }
+    Sweep S;
+    sweep_begin(P, S, L.queue);
+    bool done;
+    do {
+        const int C = sweep_next(P, S, F, L.queue, L.tab, done, cn);
+        work(C);
+    } while (!done);
+}
+
+#define RGX_TILE_LDS()                                                \
+    __shared__ int32_t s_queue[RGX_QCAP];                             \
+    __shared__ __align__(16) float s_tab[RGX_CCAP * RGX_TAB];         \
+    __shared__ uint8_t s_rowlist[4 * RGX_CCAP];                       \
+    __shared__ uint32_t s_mask[RGX_CCAP / 32][64];                    \
+    const TileLds L = {s_queue, s_tab, s_rowlist, s_mask}
+
+// lane -> pixel: row r = lane / 16 is the 4x4 block (r & 1, r >> 1) of the 8x8 tile
+__device__ __forceinline__ void lane_pixel(int px0, int py0, int &px, int &py)
+{
+    const int lane = threadIdx.x, row = lane >> 4, j = lane & 15;
+    px = px0 + (row & 1) * 4 + (j & 3);
+    py = py0 + (row >> 1) * 4 + (j >> 2);
 }
 
 // ---------------------------------------------------------------------------
@@ -510,44 +690,51 @@ __device__ __forceinline__ void frustum_range(Frustum &F, bool need, float tlo, 
 // colorBlendingT_chunked (182-203).
 __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
 {
-    __shared__ int32_t s_queue[RGX_QCAP];
-    __shared__ int32_t s_cand[RGX_CCAP];
-    __shared__ uint32_t s_mask[RGX_CCAP / 32][64];
+    RGX_TILE_LDS();
     int px0, py0;
     if (!tile_origin(P, px0, py0)) return; // whole wave
-    const int lane = threadIdx.x;
-    const int px = px0 + (lane & 7), py = py0 + (lane >> 3);
+    int px, py;
+    lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
     Counters cn;
     Frustum F;
     frustum_planes(P.cam, px0, py0, F);
     RayState R;
-    ray_begin<false>(P, px, py, valid, R, cn);
+    ray_begin<false>(P, px, py, valid, R);
     const f3 dir = R.dir;
     const int cap = P.m.max_prim_slice;
     float Cr = 0.f, Cg = 0.f, Cb = 0.f;
+    Window Wn = {0.f, 0, false, 4};
 
     while (__any(R.active)) {
         float tlo, thi;
         const bool need = slab_begin<true>(P, R, tlo, thi);
+        const bool srch = R.active && R.searching, want = need || srch;
         int p0 = 0;
         bool ov = false;
-        if (__any(need)) {
-            frustum_range(F, need, tlo, thi);
+        float found = -1.0f, searched_to = 0.f;
+        if (__any(want)) {
+            const float t0 = wave_min_all(want ? tlo : INFINITY), t1 = wave_max_all(want ? thi : -INFINITY);
+            window_ensure(P, L, F, Wn, want, tlo, R.slab_spacing, t0, t1, cn);
+            const float cover = Wn.resident ? Wn.hi : t1; // the table(s) of this iteration cover [t0, cover]
+            const float rel_hi = __any(srch) ? cover : t1;
+            const LaneQuery Q = {dir, need, tlo, thi, srch, R.tbuffer, fminf(R.texit, cover), cap};
+            searched_to = Q.shi;
             const float dt = R.dt;
-            PassState ps = {0, false};
             float sg[RGX_CHUNK_SIZE], cr[RGX_CHUNK_SIZE], cg[RGX_CHUNK_SIZE], cb[RGX_CHUNK_SIZE];
             f3 rdt;
-            auto accumulate = [&](const Prim &p, int, bool hit) {
+            auto accumulate = [&](const float4 *e, bool hit, bool) {
                 if (hit) {
-                    HitSetup hs = hit_setup(p, dir, rdt, dt);
+                    HitSetup hs = hit_setup(e, dir, rdt, dt);
+                    const float4 col = e[6];
+                    const float rho = e[4].w;
 #pragma unroll
                     for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
                         const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
-                        sg[i] = fmaf(p.rgba4.w, gw, sg[i]);
-                        cr[i] = fmaf(p.rgba4.x, gw, cr[i]);
-                        cg[i] = fmaf(p.rgba4.y, gw, cg[i]);
-                        cb[i] = fmaf(p.rgba4.z, gw, cb[i]);
+                        sg[i] = fmaf(rho, gw, sg[i]);
+                        cr[i] = fmaf(col.x, gw, cr[i]);
+                        cg[i] = fmaf(col.y, gw, cg[i]);
+                        cb[i] = fmaf(col.z, gw, cb[i]);
                         hs.power += hs.inc;
                         hs.inc += hs.inc_st;
                     }
@@ -570,7 +757,11 @@ __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
 #pragma unroll
             for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
             rdt = dir * fmaf(dt, 0.5f, R.tbuffer);
-            pass_filter(P, F, s_queue, s_cand, s_mask, ps, true, dir, need, tlo, thi, cap, p0, ov, cn, accumulate);
+            int len = 0;
+            for_each_table(P, L, F, Wn, cn, [&](int C) {
+                filter_table(L, C, t0, rel_hi, Q, p0, ov, found, len, cn);
+                shade_rows(L, len, need, accumulate);
+            });
             const bool has = need && p0 > 0;
             if (has) blend();
             // samples 16..31, only for rays still above the transmittance floor (gaussians_aabb.cu:190)
@@ -579,13 +770,18 @@ __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
 #pragma unroll
                 for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
                 rdt = dir * fmaf(dt, 16.5f, R.tbuffer);
-                if (ps.single) {
-                    pass_replay(P, s_cand, s_mask, ps, run, accumulate);
+                if (Wn.resident) {
+                    shade_rows(L, len, run, accumulate); // the row lists of the first half still stand
                 } else {
                     int q0 = 0;
                     bool qov = false;
-                    PassState ps2 = {0, false};
-                    pass_filter(P, F, s_queue, s_cand, s_mask, ps2, false, dir, run, tlo, thi, cap, q0, qov, cn, accumulate);
+                    float none = -1.0f;
+                    const LaneQuery Q2 = {dir, run, tlo, thi, false, 0.f, 0.f, cap};
+                    for_each_table(P, L, F, Wn, cn, [&](int C) {
+                        int len2;
+                        filter_table(L, C, t0, t1, Q2, q0, qov, none, len2, cn);
+                        shade_rows(L, len2, run, accumulate);
+                    });
                 }
                 if (run) blend();
             }
@@ -595,7 +791,7 @@ __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
             }
             if (ov) cn.overflow++;
         }
-        slab_end(P, R, need, p0, cn);
+        slab_end(R, need, p0, found, searched_to, cn);
     }
     if (valid) {
         const float bg = P.m.white_background ? 1.0f : 0.0f;
@@ -605,6 +801,16 @@ __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
         P.ray_colors[3 * ray + 2] = Cb + R.T * bg;
     }
     flush_stats(P.stats, cn);
+}
+
+// sum over the 16 lanes of each row, left in every lane of the row
+__device__ __forceinline__ float row_sum(float v)
+{
+    v += dpp_f<0xB1, 0xf>(0.f, v);  // quad_perm [1,0,3,2]
+    v += dpp_f<0x4E, 0xf>(0.f, v);  // quad_perm [2,3,0,1]
+    v += dpp_f<0x141, 0xf>(0.f, v); // row_half_mirror
+    v += dpp_f<0x140, 0xf>(0.f, v); // row_mirror
+    return v;
 }
 
 // ---------------------------------------------------------------------------
@@ -623,23 +829,22 @@ __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
 //   the sample point x_k = x_c + u_k dt dir (u_k = k - 15.5) is affine in k.
 // So the inner loop carries three moments (sum y, sum y u, sum y u^2) instead of
 // nineteen running sums; the `power < k^2` mask follows the reference's 32-step
-// recurrence exactly.  The 14 gradient words of a candidate are summed over the
-// lanes that hit it before they reach memory.
+// recurrence exactly.  The 14 gradient words of a Gaussian are summed over the 16
+// rays of a row with DPP adds before one lane per row adds them to memory.
 __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
 {
-    __shared__ int32_t s_queue[RGX_QCAP];
-    __shared__ int32_t s_cand[RGX_CCAP];
-    __shared__ uint32_t s_mask[RGX_CCAP / 32][64];
+    RGX_TILE_LDS();
     int px0, py0;
     if (!tile_origin(P, px0, py0)) return; // whole wave
     const int lane = threadIdx.x;
-    const int px = px0 + (lane & 7), py = py0 + (lane >> 3);
+    int px, py;
+    lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
     Counters cn;
     Frustum F;
     frustum_planes(P.cam, px0, py0, F);
     RayState R;
-    ray_begin<true>(P, px, py, valid, R, cn);
+    ray_begin<true>(P, px, py, valid, R);
     const f3 dir = R.dir;
     const int cap = P.m.max_prim_slice;
     f3 g = mk3(0.f, 0.f, 0.f);
@@ -649,46 +854,59 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
         g = mk3(P.dloss[3 * ray], P.dloss[3 * ray + 1], P.dloss[3 * ray + 2]);
         D = dot3(g, mk3(P.fwd_colors[3 * ray], P.fwd_colors[3 * ray + 1], P.fwd_colors[3 * ray + 2]));
     }
+    Window Wn = {0.f, 0, false, 4};
 
     while (__any(R.active)) {
         float tlo, thi;
         const bool need = slab_begin<false>(P, R, tlo, thi);
+        const bool srch = R.active && R.searching, want = need || srch;
         int p0 = 0;
         bool ov = false;
-        if (__any(need)) {
-            frustum_range(F, need, tlo, thi);
+        float found = -1.0f, searched_to = 0.f;
+        if (__any(want)) {
+            const float t0 = wave_min_all(want ? tlo : INFINITY), t1 = wave_max_all(want ? thi : -INFINITY);
+            window_ensure(P, L, F, Wn, want, tlo, R.slab_spacing, t0, t1, cn);
+            const float cover = Wn.resident ? Wn.hi : t1; // the table(s) of this iteration cover [t0, cover]
+            const float rel_hi = __any(srch) ? cover : t1;
+            const LaneQuery Q = {dir, need, tlo, thi, srch, R.tbuffer, fminf(R.texit, cover), cap};
+            searched_to = Q.shi;
             const float dt = R.dt, tbuffer = R.tbuffer;
-            PassState ps = {0, false};
             // (1) s_k and g.c~_k  -> PA, PB
             float PA[RGX_BUFFER_SIZE], PB[RGX_BUFFER_SIZE];
 #pragma unroll
             for (int i = 0; i < RGX_BUFFER_SIZE; ++i) PA[i] = PB[i] = 0.f;
             const f3 rdt0 = dir * fmaf(dt, 0.5f, tbuffer);
             const f3 rdt1 = dir * fmaf(dt, 16.5f, tbuffer);
-            auto densities = [&](const Prim &p, int, bool hit) {
+            auto densities = [&](const float4 *e, bool hit, bool) {
                 if (hit) {
-                    const float ddc = dot3(g, mk3(p.rgba4.x, p.rgba4.y, p.rgba4.z));
-                    HitSetup hs = hit_setup(p, dir, rdt0, dt);
+                    const float4 col = e[6];
+                    const float rho = e[4].w;
+                    const float ddc = dot3(g, mk3(col.x, col.y, col.z));
+                    HitSetup hs = hit_setup(e, dir, rdt0, dt);
 #pragma unroll
                     for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
                         const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
-                        PA[i] = fmaf(p.rgba4.w, gw, PA[i]);
+                        PA[i] = fmaf(rho, gw, PA[i]);
                         PB[i] = fmaf(ddc, gw, PB[i]);
                         hs.power += hs.inc;
                         hs.inc += hs.inc_st;
                     }
-                    hs = hit_setup(p, dir, rdt1, dt);
+                    hs = hit_setup(e, dir, rdt1, dt);
 #pragma unroll
                     for (int i = RGX_CHUNK_SIZE; i < RGX_BUFFER_SIZE; ++i) {
                         const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
-                        PA[i] = fmaf(p.rgba4.w, gw, PA[i]);
+                        PA[i] = fmaf(rho, gw, PA[i]);
                         PB[i] = fmaf(ddc, gw, PB[i]);
                         hs.power += hs.inc;
                         hs.inc += hs.inc_st;
                     }
                 }
             };
-            pass_filter(P, F, s_queue, s_cand, s_mask, ps, true, dir, need, tlo, thi, cap, p0, ov, cn, densities);
+            int len = 0;
+            for_each_table(P, L, F, Wn, cn, [&](int C) {
+                filter_table(L, C, t0, rel_hi, Q, p0, ov, found, len, cn);
+                shade_rows(L, len, need, densities);
+            });
             const bool has = need && p0 > 0;
             // (2) prefix: PA <- a_k, PB <- (T_k e_k - D_k) dt - a_k e_k   (so X_k = PB + PA * g.c_i);
             // it always covers all 32 samples (330-352)
@@ -710,24 +928,25 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
                 }
             }
             const bool use_second = T_mid > P.m.t_eps;
-            // (3) per candidate: moments per lane, wave sum, one set of atomics
+            // (3) per table entry: moments per lane, row sum, one set of atomics per row
             const f3 xdir_c = dir * fmaf(dt, 16.0f, tbuffer); // slab centre: t_c = tbuffer + 16 dt
-            auto gradients = [&](const Prim &p, int pid, bool hit) {
+            auto gradients = [&](const float4 *e, bool hit, bool live) {
                 float out[14];
 #pragma unroll
                 for (int c = 0; c < 14; ++c) out[c] = 0.f;
+                const float4 e5 = e[5];
                 if (hit) {
-                    const float k = p.inv_inter4.w;
-                    const f3 inv_s = mk3(p.inv_inter4.x * k, p.inv_inter4.y * k, p.inv_inter4.z * k);
+                    const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3], col = e[6];
+                    const float k = e2.w;
+                    const f3 inv_s = mk3(e3.x * k, e3.y * k, e3.z * k);
                     const float cut = k * k;
-                    f3 U, V, W;
-                    quat_to_cols(p.quat4, U, V, W);
-                    const float rho = p.rgba4.w;
-                    const float dcg = dot3(mk3(p.rgba4.x, p.rgba4.y, p.rgba4.z), g) / rho;
+                    const f3 U = mk3(e0.x, e0.y, e0.z), V = mk3(e1.x, e1.y, e1.z), W = mk3(e2.x, e2.y, e2.z);
+                    const float rho = e[4].w;
+                    const float dcg = dot3(mk3(col.x, col.y, col.z), g) / rho;
                     // mask recurrence exactly as backward/gaussians_aabb.cu:375-396, 437-438
                     const f3 Us = U * inv_s.x, Vs = V * inv_s.y, Ws = W * inv_s.z;
                     const f3 M1 = mk3(Us.x, Vs.x, Ws.x), M2 = mk3(Us.y, Vs.y, Ws.y), M3 = mk3(Us.z, Vs.z, Ws.z);
-                    const f3 prel = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
+                    const f3 prel = mk3(e5.x, e5.y, e5.z);
                     const f3 x0 = prel + dir * (tbuffer + 0.5f * dt);
                     const f3 Mx0 = (M1 * x0.x + M2 * x0.y) + M3 * x0.z;
                     const f3 Md = (M1 * dir.x + M2 * dir.y) + M3 * dir.z;
@@ -768,7 +987,9 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
                     out[4] = rho * dot3(M1, Vy); out[5] = rho * dot3(M2, Vy); out[6] = rho * dot3(M3, Vy); // d position
                     out[7] = rho * Sy.x * inv_s.x; out[8] = rho * Sy.y * inv_s.y; out[9] = rho * Sy.z * inv_s.z; // d scale
                     const f3 d1 = Qx * (-rho * inv_s.x), d2 = Qy * (-rho * inv_s.y), d3 = Qz * (-rho * inv_s.z); // d R columns
-                    const float qx = p.quat4.x, qy = p.quat4.y, qz = p.quat4.z, qw = p.quat4.w;
+                    // the quaternion is not in the table; fetch it (one 16-byte line per hit)
+                    const float4 q4 = P.prims[__float_as_int(e5.w)].quat4;
+                    const float qx = q4.x, qy = q4.y, qz = q4.z, qw = q4.w;
                     // backward/gaussians_aabb.cu:469-481
                     out[10] = 2 * qw * d1.y - 2 * qz * d1.z - 2 * qw * d2.x + 2 * qy * d2.z + 2 * qz * d3.x - 2 * qy * d3.y;
                     out[11] = 2 * qz * d1.y + 2 * qw * d1.z + 2 * qz * d2.x - 4 * qy * d2.y + 2 * qx * d2.z + 2 * qw * d3.x -
@@ -778,23 +999,28 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
                     out[13] = -4 * qw * d1.x + 2 * qx * d1.y + 2 * qy * d1.z - 2 * qx * d2.x - 4 * qw * d2.y + 2 * qz * d2.z +
                               2 * qy * d3.x + 2 * qz * d3.y;
                 }
-                // sum over the lanes that hit this Gaussian, then one lane adds to memory
+                const uint64_t bal = __ballot(hit);
 #pragma unroll
-                for (int c = 0; c < 14; ++c) out[c] = wave_sum_to63(out[c]);
-                if (lane == 63) {
-                    float *dst = P.gbuf + (int64_t)pid * 16;
+                for (int c = 0; c < 14; ++c) out[c] = row_sum(out[c]);
+                if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
+                    float *dst = P.gbuf + (int64_t)__float_as_int(e5.w) * 16;
 #pragma unroll
                     for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, out[c]);
                 }
             };
             if (__any(has)) {
-                if (ps.single) {
-                    pass_replay(P, s_cand, s_mask, ps, has, gradients);
+                if (Wn.resident) {
+                    shade_rows(L, len, has, gradients);
                 } else {
                     int q0 = 0;
                     bool qov = false;
-                    PassState ps2 = {0, false};
-                    pass_filter(P, F, s_queue, s_cand, s_mask, ps2, false, dir, has, tlo, thi, cap, q0, qov, cn, gradients);
+                    float none = -1.0f;
+                    const LaneQuery Q2 = {dir, has, tlo, thi, false, 0.f, 0.f, cap};
+                    for_each_table(P, L, F, Wn, cn, [&](int C) {
+                        int len2;
+                        filter_table(L, C, t0, t1, Q2, q0, qov, none, len2, cn);
+                        shade_rows(L, len2, has, gradients);
+                    });
                 }
             }
             if (has) {
@@ -805,9 +1031,51 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
             }
             if (ov) cn.overflow++;
         }
-        slab_end(P, R, need, p0, cn);
+        slab_end(R, need, p0, found, searched_to, cn);
     }
     flush_stats(P.stats, cn);
+}
+
+// Test hook for the cooperative collect: per pixel a segment [tlo, thi] (thi < tlo = pixel idle);
+// writes each ray's hit count (negated when cut at cap) and the INPUT indices of its hits.
+__global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const float *__restrict__ seg_lo,
+                                                      const float *__restrict__ seg_hi, int cap, int32_t *__restrict__ counts,
+                                                      int32_t *__restrict__ ids)
+{
+    RGX_TILE_LDS();
+    int px0, py0;
+    if (!tile_origin(P, px0, py0)) return;
+    const int lane = threadIdx.x, row = lane >> 4;
+    int px, py;
+    lane_pixel(px0, py0, px, py);
+    const bool valid = px < P.cam.width && py < P.cam.height;
+    const int64_t ray = (int64_t)py * P.cam.width + px;
+    Counters cn;
+    Frustum F;
+    frustum_planes(P.cam, px0, py0, F);
+    const f3 dir = compute_ray(P.cam, (unsigned)px, (unsigned)py);
+    const float tlo = valid ? seg_lo[ray] : 1.f, thi = valid ? seg_hi[ray] : 0.f;
+    const bool need = valid && thi >= tlo;
+    int p0 = 0, written = 0;
+    bool ov = false;
+    if (__any(need)) {
+        const float t0 = wave_min_all(need ? tlo : INFINITY), t1 = wave_max_all(need ? thi : -INFINITY);
+        Window Wn = {0.f, 0, false, 1};
+        window_ensure(P, L, F, Wn, need, tlo, 0.f, t0, t1, cn);
+        float none = -1.0f;
+        const LaneQuery Q = {dir, need, tlo, thi, false, 0.f, 0.f, cap};
+        for_each_table(P, L, F, Wn, cn, [&](int C) {
+            int len;
+            filter_table(L, C, t0, t1, Q, p0, ov, none, len, cn);
+            for (int i = 0; i < len; ++i)
+                if ((L.mask[i >> 5][lane] >> (i & 31)) & 1u) {
+                    const int c = L.rowlist[row * RGX_CCAP + i];
+                    ids[ray * cap + written++] = (int32_t)P.order[__float_as_int(L.tab[c * RGX_TAB + 23])];
+                }
+            __syncthreads();
+        });
+    }
+    if (valid) counts[ray] = ov ? -p0 : p0;
 }
 
 // gbuf (Morton order, 16 floats per Gaussian) -> the five gradient tensors in input order
@@ -861,40 +1129,6 @@ __global__ __launch_bounds__(64) void k_trace_segments(const MarchParams P, f3 o
     counts[r] = ov ? -p0 : p0;
 }
 
-
-// Test hook for the cooperative collect: per pixel a segment [tlo, thi] (thi < tlo = lane idle);
-// writes each ray's hit count (negated when cut at cap) and the INPUT indices of its hits.
-__global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const float *__restrict__ seg_lo,
-                                                      const float *__restrict__ seg_hi, int cap, int32_t *__restrict__ counts,
-                                                      int32_t *__restrict__ ids)
-{
-    __shared__ int32_t s_queue[RGX_QCAP];
-    __shared__ int32_t s_cand[RGX_CCAP];
-    __shared__ uint32_t s_mask[RGX_CCAP / 32][64];
-    int px0, py0;
-    if (!tile_origin(P, px0, py0)) return;
-    const int lane = threadIdx.x;
-    const int px = px0 + (lane & 7), py = py0 + (lane >> 3);
-    const bool valid = px < P.cam.width && py < P.cam.height;
-    const int64_t ray = (int64_t)py * P.cam.width + px;
-    Counters cn;
-    Frustum F;
-    frustum_planes(P.cam, px0, py0, F);
-    const f3 dir = compute_ray(P.cam, (unsigned)px, (unsigned)py);
-    const float tlo = valid ? seg_lo[ray] : 1.f, thi = valid ? seg_hi[ray] : 0.f;
-    const bool need = valid && thi >= tlo;
-    int p0 = 0;
-    bool ov = false;
-    if (__any(need)) {
-        frustum_range(F, need, tlo, thi);
-        PassState ps = {0, false};
-        auto record = [&](const Prim &, int pid, bool hit) {
-            if (hit) ids[ray * cap + (p0 - 1)] = (int32_t)P.order[pid];
-        };
-        pass_filter(P, F, s_queue, s_cand, s_mask, ps, false, dir, need, tlo, thi, cap, p0, ov, cn, record);
-    }
-    if (valid) counts[ray] = ov ? -p0 : p0;
-}
 
 // ---------------------------------------------------------------------------
 static inline dim3 grid_for(int64_t n, int block) { return dim3((unsigned)((n + block - 1) / block)); }

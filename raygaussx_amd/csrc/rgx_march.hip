@@ -19,6 +19,8 @@
 // hooks (arbitrary rays).
 #include "rgx_device.h"
 
+#include <type_traits>
+
 #define RGX_QCAP 1024      // node stack entries per wave (LDS)
 #define RGX_CCAP 128       // candidate table entries per wave (LDS)
 #define RGX_DFS_MARGIN 192 // above QCAP - margin the sweep pops one node at a time (depth-first)
@@ -621,53 +623,93 @@ __device__ __forceinline__ void frustum_range(Frustum &F, float t0, float t1)
     F.pad = 2.0f * RGX_PAD_REL * fmaxf(t1, 1.0f);
 }
 
-// Makes the table cover this iteration's slabs.  Returns true when the table is resident
-// (complete); false when even this iteration's own range overflows it, in which case the
-// caller walks the range in table-sized batches.
-__device__ bool window_ensure(const MarchParams &P, const TileLds &L, Frustum &F, Window &Wn, bool need, float tlo,
-                              float slab_spacing, float t0, float t1, Counters &cn)
+// One slab iteration's work on the candidate tables, in two phases that share a single copy of
+// the sweep and filter code:
+//   phase 0  make the table cover the wave's intervals (reuse the resident window, or sweep a new
+//            one looking Wn.k slabs ahead, or -- when even this iteration's own range overflows
+//            the table -- walk it in table-sized batches), filter, body_a over the row lists;
+//   mid()    per lane, between the phases; returns whether the lane takes part in phase 1;
+//   phase 1  body_b over the same row lists, or over freshly swept and filtered batches when the
+//            candidates did not fit one table.
+// Returns the phase-1 participation flag of this lane.
+template <typename BodyA, typename Mid, typename BodyB>
+__device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds &L, Frustum &F, Window &Wn, const RayState &R,
+                                            bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to,
+                                            Counters &cn, BodyA body_a, Mid mid, BodyB body_b)
 {
-    if (Wn.resident && t1 <= Wn.hi) return true;
-    for (;;) {
-        float wend = t1;
-        if (Wn.k > 1) wend = fmaxf(t1, wave_max_all(need ? tlo + (float)Wn.k * slab_spacing : -INFINITY));
-        frustum_range(F, t0, wend);
-        Sweep S;
-        sweep_begin(P, S, L.queue);
-        bool done;
-        const int C = sweep_next(P, S, F, L.queue, L.tab, done, cn);
-        if (done) {
-            Wn.hi = wend;
-            Wn.n = C;
-            Wn.resident = true;
-            if (C > (RGX_CCAP * 3) / 4) Wn.k = Wn.k > 1 ? Wn.k / 2 : 1;
-            else if (C < RGX_CCAP / 3 && Wn.k < 32) Wn.k *= 2;
-            return true;
+    const bool srch = R.active && R.searching, want = need || srch;
+    const float t0 = wave_min_all(want ? tlo : INFINITY), t1 = wave_max_all(want ? thi : -INFINITY);
+    const bool any_search = __any(srch);
+    int len = 0, q0 = 0;
+    bool run = need, qov = false;
+    for (int phase = 0; phase < 2; ++phase) {
+        const bool reuse = Wn.resident && t1 <= Wn.hi;
+        Sweep S = {0};
+        if (!reuse) {
+            float wend = t1;
+            if (phase == 0 && Wn.k > 1) wend = fmaxf(t1, wave_max_all(want ? tlo + (float)Wn.k * R.slab_spacing : -INFINITY));
+            frustum_range(F, t0, wend);
+            sweep_begin(P, S, L.queue);
         }
-        if (Wn.k == 1) break;
-        Wn.k = 1; // too many Gaussians ahead: retry with this iteration's range only
+        bool first = true, more = true;
+        while (more) {
+            int C;
+            if (reuse) {
+                C = Wn.n;
+                more = false;
+            } else {
+                bool done;
+                C = sweep_next(P, S, F, L.queue, L.tab, done, cn);
+                if (phase == 0 && first) {
+                    if (done) {
+                        Wn.hi = F.t1;
+                        Wn.n = C;
+                        Wn.resident = true;
+                        if (C > (RGX_CCAP * 3) / 4) Wn.k = Wn.k > 1 ? Wn.k / 2 : 1;
+                        else if (C < RGX_CCAP / 3 && Wn.k < 32) Wn.k *= 2;
+                    } else if (Wn.k > 1) {
+                        Wn.k = 1; // too many Gaussians ahead: start over with this iteration's range only
+                        frustum_range(F, t0, t1);
+                        sweep_begin(P, S, L.queue);
+                        continue;
+                    } else {
+                        Wn.resident = false;
+                    }
+                }
+                first = false;
+                more = !done;
+            }
+            if (phase == 0 || !Wn.resident) {
+                // phase 0 asks the lane's real question; a phase-1 re-filter only recounts the slab hits
+                const float cover = Wn.resident ? Wn.hi : t1; // this iteration's tables cover [t0, cover]
+                const LaneQuery Q = {R.dir, run, tlo, thi, phase == 0 && srch, R.tbuffer, fminf(R.texit, cover), P.m.max_prim_slice};
+                int cnt = phase == 0 ? p0 : q0;
+                bool cut = phase == 0 ? ov : qov;
+                float best = phase == 0 ? found : -1.0f;
+                filter_table(L, C, t0, (phase == 0 && any_search) ? cover : t1, Q, cnt, cut, best, len, cn);
+                if (phase == 0) {
+                    p0 = cnt;
+                    ov = cut;
+                    found = best;
+                    searched_to = Q.shi;
+                } else {
+                    q0 = cnt;
+                    qov = cut;
+                }
+            }
+            if constexpr (std::is_same<BodyA, BodyB>::value) {
+                shade_rows(L, len, run, body_a);
+            } else {
+                if (phase == 0) shade_rows(L, len, run, body_a);
+                else shade_rows(L, len, run, body_b);
+            }
+        }
+        if (phase == 0) {
+            run = mid();
+            if (!__any(run)) break;
+        }
     }
-    Wn.resident = false;
-    frustum_range(F, t0, t1);
-    return false;
-}
-
-// Runs `work(C)` on the resident table, or on each table-sized batch of a fresh sweep.
-template <typename Work>
-__device__ __forceinline__ void for_each_table(const MarchParams &P, const TileLds &L, const Frustum &F, const Window &Wn,
-                                               Counters &cn, Work work)
-{
-    if (Wn.resident) {
-        work(Wn.n);
-        return;
-    }
-    Sweep S;
-    sweep_begin(P, S, L.queue);
-    bool done;
-    do {
-        const int C = sweep_next(P, S, F, L.queue, L.tab, done, cn);
-        work(C);
-    } while (!done);
+    return run;
 }
 
 #define RGX_TILE_LDS()                                                \
@@ -702,27 +744,21 @@ __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
     RayState R;
     ray_begin<false>(P, px, py, valid, R);
     const f3 dir = R.dir;
-    const int cap = P.m.max_prim_slice;
     float Cr = 0.f, Cg = 0.f, Cb = 0.f;
     Window Wn = {0.f, 0, false, 4};
 
     while (__any(R.active)) {
         float tlo, thi;
         const bool need = slab_begin<true>(P, R, tlo, thi);
-        const bool srch = R.active && R.searching, want = need || srch;
         int p0 = 0;
         bool ov = false;
         float found = -1.0f, searched_to = 0.f;
-        if (__any(want)) {
-            const float t0 = wave_min_all(want ? tlo : INFINITY), t1 = wave_max_all(want ? thi : -INFINITY);
-            window_ensure(P, L, F, Wn, want, tlo, R.slab_spacing, t0, t1, cn);
-            const float cover = Wn.resident ? Wn.hi : t1; // the table(s) of this iteration cover [t0, cover]
-            const float rel_hi = __any(srch) ? cover : t1;
-            const LaneQuery Q = {dir, need, tlo, thi, srch, R.tbuffer, fminf(R.texit, cover), cap};
-            searched_to = Q.shi;
+        if (__any(need || (R.active && R.searching))) {
             const float dt = R.dt;
             float sg[RGX_CHUNK_SIZE], cr[RGX_CHUNK_SIZE], cg[RGX_CHUNK_SIZE], cb[RGX_CHUNK_SIZE];
-            f3 rdt;
+#pragma unroll
+            for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
+            f3 rdt = dir * fmaf(dt, 0.5f, R.tbuffer); // samples 0..15
             auto accumulate = [&](const float4 *e, bool hit, bool) {
                 if (hit) {
                     HitSetup hs = hit_setup(e, dir, rdt, dt);
@@ -753,39 +789,19 @@ __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
                     R.T *= w;
                 }
             };
-            // samples 0..15
-#pragma unroll
-            for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
-            rdt = dir * fmaf(dt, 0.5f, R.tbuffer);
-            int len = 0;
-            for_each_table(P, L, F, Wn, cn, [&](int C) {
-                filter_table(L, C, t0, rel_hi, Q, p0, ov, found, len, cn);
-                shade_rows(L, len, need, accumulate);
-            });
-            const bool has = need && p0 > 0;
-            if (has) blend();
-            // samples 16..31, only for rays still above the transmittance floor (gaussians_aabb.cu:190)
-            const bool run = has && R.T > P.m.t_eps;
-            if (__any(run)) {
+            auto second_half = [&]() {
+                const bool has = need && p0 > 0;
+                if (has) blend();
+                // samples 16..31, only for rays still above the transmittance floor (gaussians_aabb.cu:190)
 #pragma unroll
                 for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
                 rdt = dir * fmaf(dt, 16.5f, R.tbuffer);
-                if (Wn.resident) {
-                    shade_rows(L, len, run, accumulate); // the row lists of the first half still stand
-                } else {
-                    int q0 = 0;
-                    bool qov = false;
-                    float none = -1.0f;
-                    const LaneQuery Q2 = {dir, run, tlo, thi, false, 0.f, 0.f, cap};
-                    for_each_table(P, L, F, Wn, cn, [&](int C) {
-                        int len2;
-                        filter_table(L, C, t0, t1, Q2, q0, qov, none, len2, cn);
-                        shade_rows(L, len2, run, accumulate);
-                    });
-                }
-                if (run) blend();
-            }
-            if (has) {
+                return has && R.T > P.m.t_eps;
+            };
+            const bool run2 = slab_tables(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, accumulate, second_half,
+                                          accumulate);
+            if (run2) blend();
+            if (need && p0 > 0) {
                 cn.slabs++;
                 cn.hit_pairs += p0;
             }
@@ -846,7 +862,6 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
     RayState R;
     ray_begin<true>(P, px, py, valid, R);
     const f3 dir = R.dir;
-    const int cap = P.m.max_prim_slice;
     f3 g = mk3(0.f, 0.f, 0.f);
     float D = 0.f;
     if (valid) {
@@ -859,17 +874,10 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
     while (__any(R.active)) {
         float tlo, thi;
         const bool need = slab_begin<false>(P, R, tlo, thi);
-        const bool srch = R.active && R.searching, want = need || srch;
         int p0 = 0;
         bool ov = false;
         float found = -1.0f, searched_to = 0.f;
-        if (__any(want)) {
-            const float t0 = wave_min_all(want ? tlo : INFINITY), t1 = wave_max_all(want ? thi : -INFINITY);
-            window_ensure(P, L, F, Wn, want, tlo, R.slab_spacing, t0, t1, cn);
-            const float cover = Wn.resident ? Wn.hi : t1; // the table(s) of this iteration cover [t0, cover]
-            const float rel_hi = __any(srch) ? cover : t1;
-            const LaneQuery Q = {dir, need, tlo, thi, srch, R.tbuffer, fminf(R.texit, cover), cap};
-            searched_to = Q.shi;
+        if (__any(need || (R.active && R.searching))) {
             const float dt = R.dt, tbuffer = R.tbuffer;
             // (1) s_k and g.c~_k  -> PA, PB
             float PA[RGX_BUFFER_SIZE], PB[RGX_BUFFER_SIZE];
@@ -902,32 +910,31 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
                     }
                 }
             };
-            int len = 0;
-            for_each_table(P, L, F, Wn, cn, [&](int C) {
-                filter_table(L, C, t0, rel_hi, Q, p0, ov, found, len, cn);
-                shade_rows(L, len, need, densities);
-            });
-            const bool has = need && p0 > 0;
             // (2) prefix: PA <- a_k, PB <- (T_k e_k - D_k) dt - a_k e_k   (so X_k = PB + PA * g.c_i);
             // it always covers all 32 samples (330-352)
             float T_after = R.T, D_after = D;
-            float T_mid = R.T; // transmittance at the chunk boundary: gates the second chunk (398)
-            if (has) {
+            bool use_second = true; // transmittance at the chunk boundary gates the second chunk (398)
+            auto prefix = [&]() {
+                const bool has = need && p0 > 0;
+                if (has) {
+                    float T_mid = R.T;
 #pragma unroll
-                for (int i = 0; i < RGX_BUFFER_SIZE; ++i) {
-                    if (i == RGX_CHUNK_SIZE) T_mid = T_after;
-                    const float sd = PA[i];
-                    const float inv_d = sd > 0.0f ? 1.0f / sd : 0.0f;
-                    const float e = PB[i] * inv_d;
-                    const float w = __expf(-sd * dt);
-                    const float a = T_after * (1.0f - w) * inv_d;
-                    PA[i] = a;
-                    PB[i] = (T_after * e - D_after) * dt - a * e;
-                    D_after -= T_after * (1.0f - w) * e;
-                    T_after *= w;
+                    for (int i = 0; i < RGX_BUFFER_SIZE; ++i) {
+                        if (i == RGX_CHUNK_SIZE) T_mid = T_after;
+                        const float sd = PA[i];
+                        const float inv_d = sd > 0.0f ? 1.0f / sd : 0.0f;
+                        const float e = PB[i] * inv_d;
+                        const float w = __expf(-sd * dt);
+                        const float a = T_after * (1.0f - w) * inv_d;
+                        PA[i] = a;
+                        PB[i] = (T_after * e - D_after) * dt - a * e;
+                        D_after -= T_after * (1.0f - w) * e;
+                        T_after *= w;
+                    }
+                    use_second = T_mid > P.m.t_eps;
                 }
-            }
-            const bool use_second = T_mid > P.m.t_eps;
+                return has;
+            };
             // (3) per table entry: moments per lane, row sum, one set of atomics per row
             const f3 xdir_c = dir * fmaf(dt, 16.0f, tbuffer); // slab centre: t_c = tbuffer + 16 dt
             auto gradients = [&](const float4 *e, bool hit, bool live) {
@@ -1008,21 +1015,7 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
                     for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, out[c]);
                 }
             };
-            if (__any(has)) {
-                if (Wn.resident) {
-                    shade_rows(L, len, has, gradients);
-                } else {
-                    int q0 = 0;
-                    bool qov = false;
-                    float none = -1.0f;
-                    const LaneQuery Q2 = {dir, has, tlo, thi, false, 0.f, 0.f, cap};
-                    for_each_table(P, L, F, Wn, cn, [&](int C) {
-                        int len2;
-                        filter_table(L, C, t0, t1, Q2, q0, qov, none, len2, cn);
-                        shade_rows(L, len2, has, gradients);
-                    });
-                }
-            }
+            const bool has = slab_tables(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, densities, prefix, gradients);
             if (has) {
                 D = D_after;
                 R.T = T_after;
@@ -1059,21 +1052,21 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
     int p0 = 0, written = 0;
     bool ov = false;
     if (__any(need)) {
-        const float t0 = wave_min_all(need ? tlo : INFINITY), t1 = wave_max_all(need ? thi : -INFINITY);
+        RayState R;
+        R.dir = dir;
+        R.active = false; // not searching: the driver only sees the `need` lanes
+        R.searching = false;
+        R.tbuffer = tlo;
+        R.texit = thi;
+        R.slab_spacing = 0.f;
         Window Wn = {0.f, 0, false, 1};
-        window_ensure(P, L, F, Wn, need, tlo, 0.f, t0, t1, cn);
-        float none = -1.0f;
-        const LaneQuery Q = {dir, need, tlo, thi, false, 0.f, 0.f, cap};
-        for_each_table(P, L, F, Wn, cn, [&](int C) {
-            int len;
-            filter_table(L, C, t0, t1, Q, p0, ov, none, len, cn);
-            for (int i = 0; i < len; ++i)
-                if ((L.mask[i >> 5][lane] >> (i & 31)) & 1u) {
-                    const int c = L.rowlist[row * RGX_CCAP + i];
-                    ids[ray * cap + written++] = (int32_t)P.order[__float_as_int(L.tab[c * RGX_TAB + 23])];
-                }
-            __syncthreads();
-        });
+        float found = -1.0f, searched_to = 0.f;
+        MarchParams Pc = P;
+        Pc.m.max_prim_slice = cap;
+        auto record = [&](const float4 *e, bool hit, bool) {
+            if (hit) ids[ray * cap + written++] = (int32_t)P.order[__float_as_int(e[5].w)];
+        };
+        slab_tables(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, record, [] { return false; }, record);
     }
     if (valid) counts[ray] = ov ? -p0 : p0;
 }

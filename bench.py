@@ -35,9 +35,13 @@ from raygaussx_amd.render_optix import RenderOptixFunction, default_settings  # 
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per k_march_bwd launch of the default workload, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE runs scaled by a copy kernel of known size (profiles/); None until measured.
-MEASURED_TRAFFIC_BYTES = {}
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
+# script scaled by a 1 GiB copy (--calibrate-copy); the counter readings are kept in
+# profiles/march_kernels_c4_1M_800x800.md.  Workloads without a measurement report null.
+MEASURED_TRAFFIC_BYTES = {
+    ("c4_1M_800x800", "march_backward"): 9.25e9,
+    ("c4_1M_800x800", "march_forward"): 0.69e9,
+}
 
 WORKLOADS = {
     # name: (scene config, n, width, height)
@@ -75,6 +79,8 @@ def main():
     ap.add_argument("--workload", default="c4_1M_800x800", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-rays", type=int, default=1024, help="ray sample of the CPU baseline (0 = skip)")
     ap.add_argument("--forward-only", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a 1 GiB device-to-device copy (reference reading for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (--gpus 1); the path shards by views/tiles, "
@@ -82,6 +88,14 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: needs a GPU (librgx has no CPU path)")
     dev = "cuda:0"
+    if args.calibrate_copy:
+        src = torch.full((1 << 28,), 1.0, dtype=torch.float32, device=dev)     # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps(dict(calibration="copy", bytes_read=src.numel() * 4, bytes_written=dst.numel() * 4, launches=3)))
+        return
     L.lib()
     config, n, width, height = WORKLOADS[args.workload]
     cfg = dict(scenes.CONFIGS[config])

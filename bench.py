@@ -77,7 +77,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c4_1M_800x800", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-rays", type=int, default=1024, help="ray sample of the CPU baseline (0 = skip)")
+    ap.add_argument("--cpu-rays", type=int, default=16384, help="ray sample of the CPU baseline (0 = skip)")
     ap.add_argument("--forward-only", action="store_true")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy (reference reading for the FETCH_SIZE / WRITE_SIZE counters)")

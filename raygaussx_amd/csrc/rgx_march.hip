@@ -21,10 +21,18 @@
 
 #include <type_traits>
 
-#define RGX_QCAP 1024      // node stack entries per wave (LDS)
+#ifndef RGX_QCAP
+#define RGX_QCAP 448       // node stack entries per wave (LDS)
+#endif
+#ifndef RGX_CCAP
 #define RGX_CCAP 128       // candidate table entries per wave (LDS)
-#define RGX_DFS_MARGIN 192 // above QCAP - margin the sweep pops one node at a time (depth-first)
+#endif
+#define RGX_DFS_MARGIN 128 // above QCAP - margin the sweep pops one node at a time (depth-first)
 #define RGX_LDS_HITS 32    // per-lane list of the stand-alone collect hook
+// The march kernels are sized (registers and LDS) for three wavefronts per SIMD.
+#ifndef RGX_WAVES_ATTR
+#define RGX_WAVES_ATTR __attribute__((amdgpu_waves_per_eu(3, 3)))
+#endif
 
 struct MarchParams {
     RgxCamera cam;
@@ -196,6 +204,11 @@ __device__ __forceinline__ void frustum_planes(const RgxCamera &cam, int px0, in
     F.n[1] = plane_normal(d10, d11, in);
     F.n[2] = plane_normal(d00, d10, in);
     F.n[3] = plane_normal(d01, d11, in);
+    // the planes are the same in every lane: keep them in scalar registers
+    auto uni = [](float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); };
+    F.o = mk3(uni(F.o.x), uni(F.o.y), uni(F.o.z));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) F.n[k] = mk3(uni(F.n[k].x), uni(F.n[k].y), uni(F.n[k].z));
 }
 
 __device__ __forceinline__ bool frustum_overlaps(const Frustum &F, float4 a, float4 b)
@@ -226,8 +239,10 @@ __device__ __forceinline__ bool frustum_overlaps(const Frustum &F, float4 a, flo
 // from the eye that bounds the ellipsoid.  The values are produced by the same operations,
 // in the same order, as in line_roots(), so using them changes no rounding.
 //   float4 0: U.xyz, dmin     1: V.xyz, dmax     2: W.xyz, k      3: inv_inter.xyz, c
-//          4: Oe.xyz, rho     5: (eye-centre).xyz, sorted index   6: rgb*rho, -
-#define RGX_TAB 28
+//          4: Oe.xyz, sorted index
+// (80 bytes, sized so that 12 wavefronts' tables fit one CU's LDS; what only the shading of an
+// actual hit needs -- eye - centre and the colour -- is read from the primitive record.)
+#define RGX_TAB 20
 
 // Cooperative sweep of the BVH: the node stack is shared by the wave, every step pops up to
 // 64 nodes (one per lane) and tests their boxes against the frustum.  Internal nodes that pass
@@ -274,19 +289,20 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
             }
         }
         if (lane == 0) cn.nodes += (unsigned)m;
-        float4 e[7];
+        // leaf: test the actual ellipsoid, then (after the wave has agreed on table slots) write the entry
+        Prim p;
+        f3 U, V, W;
+        float dmin = 0.f, dmax = 0.f;
         if (leaf_hit) {
-            const int32_t pid = ~left;
-            const Prim p = P.prims[pid];
-            f3 U, V, W;
+            p = P.prims[~left];
             quat_to_cols(p.quat4, U, V, W);
-            const f3 inv = mk3(p.inv_inter4.x, p.inv_inter4.y, p.inv_inter4.z);
             const f3 O = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
             // semi-axes of the k-sigma ellipsoid: k * scale = 1 / inv_inter
-            const f3 ax = mk3(1.0f / inv.x, 1.0f / inv.y, 1.0f / inv.z);
+            const f3 ax = mk3(1.0f / p.inv_inter4.x, 1.0f / p.inv_inter4.y, 1.0f / p.inv_inter4.z);
             const float dist = sqrtf(dot3(O, O));
             const float rad = fmaxf(ax.x, fmaxf(ax.y, ax.z)) * 1.001f + 1e-5f * dist + F.pad;
-            const float dmin = dist - rad, dmax = dist + rad;
+            dmin = dist - rad;
+            dmax = dist + rad;
             bool ok = p.inv_inter4.w == p.inv_inter4.w; // k is NaN below the density threshold: never hit
             ok = ok && dmax >= F.t0 && dmin <= F.t1;
 #pragma unroll
@@ -298,21 +314,18 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
                 ok = ok && !(-dot3(n, O) - h > F.pad);
             }
             leaf_hit = ok;
-            const f3 Oe = apply_sinv_rt(O, U, V, W, inv);
-            const float cc = fmaf(Oe.x, Oe.x, fmaf(Oe.y, Oe.y, fmaf(Oe.z, Oe.z, -1.0f)));
-            e[0] = make_float4(U.x, U.y, U.z, dmin);
-            e[1] = make_float4(V.x, V.y, V.z, dmax);
-            e[2] = make_float4(W.x, W.y, W.z, p.inv_inter4.w);
-            e[3] = make_float4(inv.x, inv.y, inv.z, cc);
-            e[4] = make_float4(Oe.x, Oe.y, Oe.z, p.rgba4.w);
-            e[5] = make_float4(O.x, O.y, O.z, __int_as_float(pid));
-            e[6] = make_float4(p.rgba4.x, p.rgba4.y, p.rgba4.z, 0.f);
         }
         const uint64_t bl = __ballot(leaf_hit), bi = __ballot(inner_hit);
         if (leaf_hit) {
             float4 *dst = (float4 *)(s_tab + (C + __popcll(bl & lt)) * RGX_TAB);
-#pragma unroll
-            for (int k = 0; k < 7; ++k) dst[k] = e[k];
+            const f3 inv = mk3(p.inv_inter4.x, p.inv_inter4.y, p.inv_inter4.z);
+            const f3 O = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
+            dst[0] = make_float4(U.x, U.y, U.z, dmin);
+            dst[1] = make_float4(V.x, V.y, V.z, dmax);
+            dst[2] = make_float4(W.x, W.y, W.z, p.inv_inter4.w);
+            const f3 Oe = apply_sinv_rt(O, U, V, W, inv);
+            dst[3] = make_float4(inv.x, inv.y, inv.z, fmaf(Oe.x, Oe.x, fmaf(Oe.y, Oe.y, fmaf(Oe.z, Oe.z, -1.0f))));
+            dst[4] = make_float4(Oe.x, Oe.y, Oe.z, __int_as_float(~left));
         }
         C += __popcll(bl);
         if (inner_hit) {
@@ -495,9 +508,9 @@ __device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, f
 struct HitSetup {
     float power, inc, inc_st, cut;
 };
-__device__ __forceinline__ HitSetup hit_setup(const float4 *e, f3 dir, f3 ray_dir_tmid, float dt)
+__device__ __forceinline__ HitSetup hit_setup(const float4 *e, float4 e5, f3 dir, f3 ray_dir_tmid, float dt)
 {
-    const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3], e5 = e[5];
+    const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3]; // e5 = pos4 of the primitive: eye - centre
     const float k = e2.w;
     const f3 inv_s = mk3(e3.x * k, e3.y * k, e3.z * k);
     const f3 U = mk3(e0.x, e0.y, e0.z), V = mk3(e1.x, e1.y, e1.z), W = mk3(e2.x, e2.y, e2.z);
@@ -730,7 +743,7 @@ __device__ __forceinline__ void lane_pixel(int px0, int py0, int &px, int &py)
 // ---------------------------------------------------------------------------
 // Forward: __raygen__rg (gaussians_aabb.cu:205-340), accumulateChunk (112-180),
 // colorBlendingT_chunked (182-203).
-__global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchParams P)
 {
     RGX_TILE_LDS();
     int px0, py0;
@@ -761,9 +774,10 @@ __global__ __launch_bounds__(64) void k_march_fwd(const MarchParams P)
             f3 rdt = dir * fmaf(dt, 0.5f, R.tbuffer); // samples 0..15
             auto accumulate = [&](const float4 *e, bool hit, bool) {
                 if (hit) {
-                    HitSetup hs = hit_setup(e, dir, rdt, dt);
-                    const float4 col = e[6];
-                    const float rho = e[4].w;
+                    const Prim *pr = P.prims + __float_as_int(e[4].w);
+                    const float4 col = pr->rgba4;
+                    HitSetup hs = hit_setup(e, pr->pos4, dir, rdt, dt);
+                    const float rho = col.w;
 #pragma unroll
                     for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
                         const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
@@ -847,7 +861,7 @@ __device__ __forceinline__ float row_sum(float v)
 // nineteen running sums; the `power < k^2` mask follows the reference's 32-step
 // recurrence exactly.  The 14 gradient words of a Gaussian are summed over the 16
 // rays of a row with DPP adds before one lane per row adds them to memory.
-__global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchParams P)
 {
     RGX_TILE_LDS();
     int px0, py0;
@@ -887,10 +901,11 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
             const f3 rdt1 = dir * fmaf(dt, 16.5f, tbuffer);
             auto densities = [&](const float4 *e, bool hit, bool) {
                 if (hit) {
-                    const float4 col = e[6];
-                    const float rho = e[4].w;
+                    const Prim *pr = P.prims + __float_as_int(e[4].w);
+                    const float4 col = pr->rgba4, pos4 = pr->pos4;
+                    const float rho = col.w;
                     const float ddc = dot3(g, mk3(col.x, col.y, col.z));
-                    HitSetup hs = hit_setup(e, dir, rdt0, dt);
+                    HitSetup hs = hit_setup(e, pos4, dir, rdt0, dt);
 #pragma unroll
                     for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
                         const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
@@ -899,7 +914,7 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
                         hs.power += hs.inc;
                         hs.inc += hs.inc_st;
                     }
-                    hs = hit_setup(e, dir, rdt1, dt);
+                    hs = hit_setup(e, pos4, dir, rdt1, dt);
 #pragma unroll
                     for (int i = RGX_CHUNK_SIZE; i < RGX_BUFFER_SIZE; ++i) {
                         const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
@@ -941,14 +956,15 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
                 float out[14];
 #pragma unroll
                 for (int c = 0; c < 14; ++c) out[c] = 0.f;
-                const float4 e5 = e[5];
+                const int32_t pid = __float_as_int(e[4].w);
                 if (hit) {
-                    const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3], col = e[6];
+                    const Prim *pr = P.prims + pid;
+                    const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3], col = pr->rgba4, e5 = pr->pos4;
                     const float k = e2.w;
                     const f3 inv_s = mk3(e3.x * k, e3.y * k, e3.z * k);
                     const float cut = k * k;
                     const f3 U = mk3(e0.x, e0.y, e0.z), V = mk3(e1.x, e1.y, e1.z), W = mk3(e2.x, e2.y, e2.z);
-                    const float rho = e[4].w;
+                    const float rho = col.w;
                     const float dcg = dot3(mk3(col.x, col.y, col.z), g) / rho;
                     // mask recurrence exactly as backward/gaussians_aabb.cu:375-396, 437-438
                     const f3 Us = U * inv_s.x, Vs = V * inv_s.y, Ws = W * inv_s.z;
@@ -994,8 +1010,7 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
                     out[4] = rho * dot3(M1, Vy); out[5] = rho * dot3(M2, Vy); out[6] = rho * dot3(M3, Vy); // d position
                     out[7] = rho * Sy.x * inv_s.x; out[8] = rho * Sy.y * inv_s.y; out[9] = rho * Sy.z * inv_s.z; // d scale
                     const f3 d1 = Qx * (-rho * inv_s.x), d2 = Qy * (-rho * inv_s.y), d3 = Qz * (-rho * inv_s.z); // d R columns
-                    // the quaternion is not in the table; fetch it (one 16-byte line per hit)
-                    const float4 q4 = P.prims[__float_as_int(e5.w)].quat4;
+                    const float4 q4 = pr->quat4;
                     const float qx = q4.x, qy = q4.y, qz = q4.z, qw = q4.w;
                     // backward/gaussians_aabb.cu:469-481
                     out[10] = 2 * qw * d1.y - 2 * qz * d1.z - 2 * qw * d2.x + 2 * qy * d2.z + 2 * qz * d3.x - 2 * qy * d3.y;
@@ -1010,7 +1025,7 @@ __global__ __launch_bounds__(64) void k_march_bwd(const MarchParams P)
 #pragma unroll
                 for (int c = 0; c < 14; ++c) out[c] = row_sum(out[c]);
                 if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
-                    float *dst = P.gbuf + (int64_t)__float_as_int(e5.w) * 16;
+                    float *dst = P.gbuf + (int64_t)pid * 16;
 #pragma unroll
                     for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, out[c]);
                 }
@@ -1064,7 +1079,7 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
         MarchParams Pc = P;
         Pc.m.max_prim_slice = cap;
         auto record = [&](const float4 *e, bool hit, bool) {
-            if (hit) ids[ray * cap + written++] = (int32_t)P.order[__float_as_int(e[5].w)];
+            if (hit) ids[ray * cap + written++] = (int32_t)P.order[__float_as_int(e[4].w)];
         };
         slab_tables(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, record, [] { return false; }, record);
     }

@@ -79,6 +79,8 @@ def main():
     ap.add_argument("--workload", default="c4_1M_800x800", choices=sorted(WORKLOADS))
     ap.add_argument("--cpu-rays", type=int, default=16384, help="ray sample of the CPU baseline (0 = skip)")
     ap.add_argument("--forward-only", action="store_true")
+    ap.add_argument("--no-records", action="store_true",
+                    help="backward searches the tree again instead of replaying the forward's hit-list record")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy (reference reading for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -116,6 +118,7 @@ def main():
         s = default_settings(cams[i % n_cams], cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
                              t_eps=cfg["t_eps"], gas=gas)
         s.stats = stats
+        s.record_hits = not args.no_records
         img = RenderOptixFunction.apply(*params, s)
         gas = s.gas
         if not args.forward_only:

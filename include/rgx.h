@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define RGX_ABI_VERSION 1
+#define RGX_ABI_VERSION 2
 
 #define RGX_OK 0
 #define RGX_EINVAL -1     /* bad argument (null pointer, negative size, unsupported degree ...) */
@@ -68,6 +68,7 @@ typedef struct RgxStats {
     unsigned long long nodes_visited; /* BVH nodes fetched by all queries */
     unsigned long long candidates;     /* Gaussians gathered per tile and slab iteration (filter passes) */
     unsigned long long candidates_hit; /* ... of which at least one ray of the tile hit */
+    unsigned long long replay_lost;    /* tiles whose backward did not consume its hit-list record exactly (expect 0) */
 } RgxStats;
 
 int rgx_abi_version(void);
@@ -132,26 +133,37 @@ int rgx_pack_prims(const void *ws, const float *eye, const float *pos, const flo
 /* ---- ray march ------------------------------------------------------------ */
 
 /* Scratch for one march launch: the backward's Morton-ordered gradient block.  (The
- * reference's per-ray hit scratch hit_prim_idx, optix_utils.py:306, has no counterpart:
- * hit lists never leave the chip.) */
+ * reference's per-ray hit scratch hit_prim_idx, optix_utils.py:306, has no counterpart.) */
 int rgx_march_workspace_bytes(int64_t n, int64_t n_rays, int32_t max_prim_slice, size_t *bytes);
+
+/* Optional hit-list record of one forward launch: per 8x8 pixel tile a region of tile_words
+ * 32-bit words (>= 1024, multiple of 4; 16384 is ample for the benchmark scenes) holding, per
+ * slab iteration, which Gaussians each 4x4 pixel row hits and each ray's hit bits.  A backward
+ * given the record of its forward replays those lists instead of searching the tree again;
+ * tiles whose region overflowed are recomputed.  The role the reference's hit_prim_idx buffer
+ * plays between its collect and blend steps (optix_utils.py:306), at a few hundred bytes per
+ * tile and slab instead of max_prim_slice ints per ray. */
+int rgx_march_records_bytes(int32_t width, int32_t height, int32_t tile_words, size_t *bytes);
 
 /* Replaces launch_pipeline_forward / launch_pipeline_test (optix_utils.py:222-322,
  * 503-601) and the OptiX programs of cuda_train/forward/gaussians_aabb.cu:
  * ray_colors (W*H,3), row-major pixels.  cam, march: host structs.
- * prims: from rgx_pack_prims with the same ws.  stats may be NULL. */
+ * prims: from rgx_pack_prims with the same ws.  records (16-byte aligned, may be NULL):
+ * where to write the hit-list record.  stats may be NULL. */
 int rgx_march_forward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims,
                       int64_t n, float *ray_colors, void *march_ws, size_t march_ws_bytes,
-                      RgxStats *stats, void *stream);
+                      void *records, size_t records_bytes, RgxStats *stats, void *stream);
 
 /* Replaces launch_pipeline_backward + reduce_temp_grads (optix_utils.py:325-500) and
  * cuda_train/backward/gaussians_aabb.cu: gradients of sum(dloss * ray_colors) with
  * respect to density (N), rgb (N,3), position (N,3), scale (N,3), quaternion (N,4),
- * in INPUT order, overwritten.  ray_colors is the forward's output. */
+ * in INPUT order, overwritten.  ray_colors is the forward's output.  records: the record
+ * written by the forward launch with the same ws, cam, march and prims, or NULL. */
 int rgx_march_backward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims,
                        int64_t n, const float *ray_colors, const float *dloss, float *ddens,
                        float *drgb, float *dpos, float *dscale, float *dquat, void *march_ws,
-                       size_t march_ws_bytes, RgxStats *stats, void *stream);
+                       size_t march_ws_bytes, const void *records, size_t records_bytes,
+                       RgxStats *stats, void *stream);
 
 /* Test hooks: the two OptiX ray queries on caller-supplied segments (origin = eye,
  * host float[3]; dirs (n,3); tlo/thi (n)).  first-hit: optixTrace SBT offset 0

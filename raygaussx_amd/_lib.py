@@ -29,12 +29,14 @@ class RgxMarch(C.Structure):
 
 
 STATS_FIELDS = ("hit_pairs", "slabs", "empty_slabs", "overflow_rays", "rays_hit", "nodes_visited", "candidates",
-                "candidates_hit")
+                "candidates_hit", "replay_lost")
+
+ABI_VERSION = 2   # RGX_ABI_VERSION of include/rgx.h
 
 # every symbol include/rgx.h declares
 SYMBOLS = ("rgx_abi_version", "rgx_strerror", "rgx_last_hip_error", "rgx_aabb", "rgx_sh_forward",
            "rgx_sh_backward", "rgx_build_workspace_bytes", "rgx_build", "rgx_build_aabbs", "rgx_scene_bbox",
-           "rgx_build_order", "rgx_pack_prims", "rgx_march_workspace_bytes", "rgx_march_forward",
+           "rgx_build_order", "rgx_pack_prims", "rgx_march_workspace_bytes", "rgx_march_records_bytes", "rgx_march_forward",
            "rgx_march_backward", "rgx_first_hit", "rgx_trace_segments", "rgx_collect_tiles", "rgx_morton_workspace_bytes",
            "rgx_morton_order", "rgx_timing_enable", "rgx_timing_reset", "rgx_timing_name", "rgx_timing_read")
 
@@ -52,6 +54,9 @@ def lib():
         _lib.rgx_timing_name.restype = C.c_char_p
         for name in SYMBOLS:
             getattr(_lib, name)  # fail at load time if the library is stale
+        if _lib.rgx_abi_version() != ABI_VERSION:
+            got, _lib = _lib.rgx_abi_version(), None
+            raise RgxError(f"{LIB_PATH} has ABI version {got}, this binding needs {ABI_VERSION}; rebuild it")
     return _lib
 
 

@@ -49,12 +49,16 @@ struct MarchParams {
     float *gbuf;             // bwd: (n,16) gradient block in Morton order
     RgxStats *stats;
     int32_t tiles_x, tiles_y;
+    uint32_t *records;      // hit-list record stream, rec_tile_words per tile, or null
+    int32_t rec_tile_words;
+    int32_t only_overflow;  // backward: handle only the tiles whose record overflowed
 };
 
 struct Counters {
     unsigned hit_pairs = 0, slabs = 0, empty = 0, overflow = 0, rays_hit = 0;
     unsigned long long nodes = 0;
     unsigned cands = 0, cands_hit = 0; // per wave (lane 0 counts)
+    unsigned replay_lost = 0;          // per wave: the backward's replay did not consume its record exactly
 };
 
 // ---------------------------------------------------------------------------
@@ -343,7 +347,7 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
     return C;
 }
 
-__device__ __forceinline__ bool tile_origin(const MarchParams &P, int &px0, int &py0)
+__device__ __forceinline__ bool tile_origin(const MarchParams &P, int &px0, int &py0, int *tile_out = nullptr)
 {
     // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one contiguous
     // band of tiles so its L2 sees one region of the scene.
@@ -352,14 +356,15 @@ __device__ __forceinline__ bool tile_origin(const MarchParams &P, int &px0, int 
     const int tile = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
     px0 = (tile % P.tiles_x) * 8;
     py0 = (tile / P.tiles_x) * 8;
+    if (tile_out) *tile_out = tile;
     return tile < ntiles;
 }
 
 __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
 {
     if (!st) return;
-    unsigned long long v[8] = {c.hit_pairs, c.slabs, c.empty, c.overflow, c.rays_hit, c.nodes, c.cands, c.cands_hit};
-    for (int k = 0; k < 8; ++k) {
+    unsigned long long v[9] = {c.hit_pairs, c.slabs, c.empty, c.overflow, c.rays_hit, c.nodes, c.cands, c.cands_hit, c.replay_lost};
+    for (int k = 0; k < 9; ++k) {
         unsigned long long x = v[k];
         for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
         v[k] = x;
@@ -368,6 +373,7 @@ __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
         atomicAdd(&st->hit_pairs, v[0]); atomicAdd(&st->slabs, v[1]); atomicAdd(&st->empty_slabs, v[2]);
         atomicAdd(&st->overflow_rays, v[3]); atomicAdd(&st->rays_hit, v[4]); atomicAdd(&st->nodes_visited, v[5]);
         atomicAdd(&st->candidates, v[6]); atomicAdd(&st->candidates_hit, v[7]);
+        if (v[8]) atomicAdd(&st->replay_lost, v[8]);
     }
 }
 
@@ -504,17 +510,38 @@ __device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, f
     return true;
 }
 
-// Per-hit constants of the sample recurrence (gaussians_aabb.cu:135-164), from a table entry.
+// A Gaussian as the shading code sees it: its record in HBM plus its rotation columns,
+// inverse scales / k and k -- read from the LDS table entry when there is one, recomputed
+// from the record (same operations, same values) when a recorded hit list is replayed.
+template <bool FROM_TABLE>
+struct Entry {
+    const float4 *tab; // LDS table entry (FROM_TABLE only)
+    const Prim *prim;
+    int32_t pid;       // index in Morton order
+    __device__ __forceinline__ void frame(f3 &U, f3 &V, f3 &W, f3 &inv, float &k) const
+    {
+        if constexpr (FROM_TABLE) {
+            const float4 e0 = tab[0], e1 = tab[1], e2 = tab[2], e3 = tab[3];
+            U = mk3(e0.x, e0.y, e0.z); V = mk3(e1.x, e1.y, e1.z); W = mk3(e2.x, e2.y, e2.z);
+            inv = mk3(e3.x, e3.y, e3.z);
+            k = e2.w;
+        } else {
+            const float4 q = prim->quat4, i4 = prim->inv_inter4;
+            quat_to_cols(q, U, V, W);
+            inv = mk3(i4.x, i4.y, i4.z);
+            k = i4.w;
+        }
+    }
+};
+
+// Per-hit constants of the sample recurrence (gaussians_aabb.cu:135-164).
 struct HitSetup {
     float power, inc, inc_st, cut;
 };
-__device__ __forceinline__ HitSetup hit_setup(const float4 *e, float4 e5, f3 dir, f3 ray_dir_tmid, float dt)
+__device__ __forceinline__ HitSetup hit_setup(f3 U, f3 V, f3 W, f3 inv, float k, float4 pos4, f3 dir, f3 ray_dir_tmid, float dt)
 {
-    const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3]; // e5 = pos4 of the primitive: eye - centre
-    const float k = e2.w;
-    const f3 inv_s = mk3(e3.x * k, e3.y * k, e3.z * k);
-    const f3 U = mk3(e0.x, e0.y, e0.z), V = mk3(e1.x, e1.y, e1.z), W = mk3(e2.x, e2.y, e2.z);
-    const f3 xhit = mk3(e5.x, e5.y, e5.z) + ray_dir_tmid;
+    const f3 inv_s = mk3(inv.x * k, inv.y * k, inv.z * k);
+    const f3 xhit = mk3(pos4.x, pos4.y, pos4.z) + ray_dir_tmid;
     const f3 Mx0 = apply_sinv_rt(xhit, U, V, W, inv_s);
     const f3 Md = apply_sinv_rt(dir, U, V, W, inv_s);
     const float Md2 = dot3(Md, Md);
@@ -549,9 +576,6 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
     const int lane = threadIdx.x, row = lane >> 4;
     len = 0;
     uint32_t bits = 0;
-#ifdef RGX_EXP_NOFILTER
-    if (C >= 0) { p0 = 1; return; }
-#endif
     for (int h = 0; h < RGX_CCAP / 64; ++h) {
         const int cl = h * 64 + lane;
         bool rel = false;
@@ -599,25 +623,122 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
 // Shade: the four rows walk their own lists in lock step; body(entry, hit, live) runs whenever
 // some lane hits (hit: this lane hits this entry; live: this lane's row still has an entry at i).
 template <typename Body>
-__device__ __forceinline__ void shade_rows(const TileLds &L, int len, bool run, Body body)
+__device__ __forceinline__ void shade_rows(const MarchParams &P, const TileLds &L, int len, bool run, Body body)
 {
     const int lane = threadIdx.x, row = lane >> 4;
     const int l0 = __builtin_amdgcn_readlane(len, 0), l1 = __builtin_amdgcn_readlane(len, 16);
     const int l2 = __builtin_amdgcn_readlane(len, 32), l3 = __builtin_amdgcn_readlane(len, 48);
     const int maxlen = max(max(l0, l1), max(l2, l3));
     uint32_t bits = 0;
-#ifdef RGX_EXP_NOSHADE
-    if (maxlen >= 0) return;
-#endif
     for (int i = 0; i < maxlen; ++i) {
         if ((i & 31) == 0) bits = L.mask[i >> 5][lane];
         const bool live = i < len;
         const bool hit = run && live && ((bits >> (i & 31)) & 1u);
         if (__ballot(hit)) {
             const int c = live ? L.rowlist[row * RGX_CCAP + i] : 0;
-            body((const float4 *)(L.tab + c * RGX_TAB), hit, live);
+            const float4 *tab = (const float4 *)(L.tab + c * RGX_TAB);
+            const int32_t pid = __float_as_int(L.tab[c * RGX_TAB + 19]);
+            body(Entry<true>{tab, P.prims + pid, pid}, hit, live);
         }
     }
+}
+
+// ---------------------------------------------------------------------------
+// Hit-list records.  What the filter produces for a slab iteration -- per 4x4 row the Gaussians
+// some ray of the row hits, per ray its hit bits over that list, per searching ray the first-hit
+// t -- is a few hundred bytes.  The forward can stream it to memory so that the backward replays
+// the same lists instead of sweeping the tree and evaluating the predicate again; within one
+// kernel the same records let the second pass of an iteration whose candidates did not fit one
+// table skip its second sweep.  Per tile a region of rec_tile_words 32-bit words:
+//   word 0: 0 = complete, 1 = the region overflowed (record unusable);  word 1: words used;
+//   from word 4, per iteration:  one LISTS item per table batch, then a TRAIL item
+//   LISTS: {tag | last << 8 | nw, len[4], -, -, -}, pid[pad4(len[r])] for r = 0..3, mask[nw][64]
+//   TRAIL: {tag | any_search, cover (float), -, -}, found[64] when any_search
+#define RGX_REC_LISTS 0x4C000000u
+#define RGX_REC_TRAIL 0x54000000u
+
+struct Recorder {
+    uint32_t *reg;  // this tile's region, or null
+    int off;        // next free word (wave-uniform)
+    int cap;        // words in the region
+    bool ovf;       // the region is exhausted
+    int iter_start; // first item of the current iteration
+    __device__ __forceinline__ bool on() const { return reg != nullptr && !ovf; }
+
+    __device__ __forceinline__ void write_lists(const TileLds &L, int len, bool last)
+    {
+        if (!on()) return;
+        const int lane = threadIdx.x, row = lane >> 4;
+        const int l0 = __builtin_amdgcn_readlane(len, 0), l1 = __builtin_amdgcn_readlane(len, 16);
+        const int l2 = __builtin_amdgcn_readlane(len, 32), l3 = __builtin_amdgcn_readlane(len, 48);
+        const int nw = (max(max(l0, l1), max(l2, l3)) + 31) >> 5;
+        const int p0 = (l0 + 3) & ~3, p1 = (l1 + 3) & ~3, p2 = (l2 + 3) & ~3, p3 = (l3 + 3) & ~3;
+        const int size = 8 + p0 + p1 + p2 + p3 + nw * 64;
+        if (off + size + 72 > cap) { // always leave room for the iteration's trailer
+            ovf = true;
+            return;
+        }
+        uint32_t *it = reg + off;
+        if (lane == 0) {
+            it[0] = RGX_REC_LISTS | (last ? 0x100u : 0u) | (uint32_t)nw;
+            it[1] = (uint32_t)l0; it[2] = (uint32_t)l1; it[3] = (uint32_t)l2; it[4] = (uint32_t)l3;
+        }
+        const int base = 8 + (row > 0 ? p0 : 0) + (row > 1 ? p1 : 0) + (row > 2 ? p2 : 0);
+        for (int i = lane & 15; i < len; i += 16)
+            it[base + i] = __float_as_uint(L.tab[L.rowlist[row * RGX_CCAP + i] * RGX_TAB + 19]);
+        const int mbase = 8 + p0 + p1 + p2 + p3;
+        for (int w = 0; w < nw; ++w) it[mbase + w * 64 + lane] = L.mask[w][lane];
+        off += size;
+    }
+
+    __device__ __forceinline__ void write_trailer(bool any_search, float cover, float found)
+    {
+        if (!on()) return;
+        uint32_t *it = reg + off;
+        if (threadIdx.x == 0) {
+            it[0] = RGX_REC_TRAIL | (any_search ? 1u : 0u);
+            it[1] = __float_as_uint(cover);
+        }
+        if (any_search) it[4 + threadIdx.x] = __float_as_uint(found);
+        off += 4 + (any_search ? 64 : 0);
+    }
+
+    __device__ __forceinline__ void finish()
+    {
+        if (reg && threadIdx.x == 0) {
+            reg[0] = ovf ? 1u : 0u;
+            reg[1] = (uint32_t)off;
+        }
+    }
+};
+
+__device__ __forceinline__ uint32_t uni_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+
+// Replays one LISTS item: the four rows walk their recorded lists in lock step, exactly as
+// shade_rows does on a live table.  COUNT adds the lane's hits to p0.  Returns the item's size.
+template <bool COUNT, typename Body>
+__device__ __forceinline__ int replay_lists(const MarchParams &P, const uint32_t *it, bool run, int &p0, Body body)
+{
+    const int lane = threadIdx.x, row = lane >> 4;
+    const int nw = (int)(uni_u32(it[0]) & 0xffu);
+    const int l0 = (int)uni_u32(it[1]), l1 = (int)uni_u32(it[2]), l2 = (int)uni_u32(it[3]), l3 = (int)uni_u32(it[4]);
+    const int q0 = (l0 + 3) & ~3, q1 = (l1 + 3) & ~3, q2 = (l2 + 3) & ~3, q3 = (l3 + 3) & ~3;
+    const int len = row == 0 ? l0 : row == 1 ? l1 : row == 2 ? l2 : l3;
+    const uint32_t *pids = it + 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0);
+    const uint32_t *masks = it + 8 + q0 + q1 + q2 + q3;
+    const int maxlen = max(max(l0, l1), max(l2, l3));
+    uint32_t bits = 0;
+    for (int i = 0; i < maxlen; ++i) {
+        if ((i & 31) == 0) bits = masks[(i >> 5) * 64 + lane];
+        const bool live = i < len;
+        const bool hit = run && live && ((bits >> (i & 31)) & 1u);
+        if (COUNT && hit) ++p0;
+        if (__ballot(hit)) {
+            const int32_t pid = live ? (int32_t)pids[i] : 0;
+            body(Entry<false>{nullptr, P.prims + pid, pid}, hit, live);
+        }
+    }
+    return 8 + q0 + q1 + q2 + q3 + nw * 64;
 }
 
 // Resident candidate window: the table holds every Gaussian of the tile frustum between the
@@ -648,14 +769,25 @@ __device__ __forceinline__ void frustum_range(Frustum &F, float t0, float t1)
 template <typename BodyA, typename Mid, typename BodyB>
 __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds &L, Frustum &F, Window &Wn, const RayState &R,
                                             bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to,
-                                            Counters &cn, BodyA body_a, Mid mid, BodyB body_b)
+                                            Counters &cn, Recorder &rec, BodyA body_a, Mid mid, BodyB body_b)
 {
     const bool srch = R.active && R.searching, want = need || srch;
+    rec.iter_start = rec.off;
     const float t0 = wave_min_all(want ? tlo : INFINITY), t1 = wave_max_all(want ? thi : -INFINITY);
     const bool any_search = __any(srch);
     int len = 0, q0 = 0;
     bool run = need, qov = false;
     for (int phase = 0; phase < 2; ++phase) {
+        if (phase == 1 && !Wn.resident && rec.on()) {
+            // the batches of this iteration were recorded: replay them instead of sweeping again
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+            __syncthreads();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+            int at = rec.iter_start, dummy = 0;
+            while (at < rec.off && (uni_u32(rec.reg[at]) & 0xff000000u) == RGX_REC_LISTS)
+                at += replay_lists<false>(P, rec.reg + at, run, dummy, body_b);
+            break;
+        }
         const bool reuse = Wn.resident && t1 <= Wn.hi;
         Sweep S = {0};
         if (!reuse) {
@@ -705,22 +837,64 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                     ov = cut;
                     found = best;
                     searched_to = Q.shi;
+                    rec.write_lists(L, len, !more);
                 } else {
                     q0 = cnt;
                     qov = cut;
                 }
             }
             if constexpr (std::is_same<BodyA, BodyB>::value) {
-                shade_rows(L, len, run, body_a);
+                shade_rows(P, L, len, run, body_a);
             } else {
-                if (phase == 0) shade_rows(L, len, run, body_a);
-                else shade_rows(L, len, run, body_b);
+                if (phase == 0) shade_rows(P, L, len, run, body_a);
+                else shade_rows(P, L, len, run, body_b);
             }
         }
         if (phase == 0) {
+            rec.write_trailer(any_search, Wn.resident ? Wn.hi : t1, found);
             run = mid();
             if (!__any(run)) break;
         }
+    }
+    return run;
+}
+
+// Size in words of the LISTS item at `it`.
+__device__ __forceinline__ int lists_size(const uint32_t *it)
+{
+    const int nw = (int)(uni_u32(it[0]) & 0xffu);
+    const int l0 = (int)uni_u32(it[1]), l1 = (int)uni_u32(it[2]), l2 = (int)uni_u32(it[3]), l3 = (int)uni_u32(it[4]);
+    return 8 + ((l0 + 3) & ~3) + ((l1 + 3) & ~3) + ((l2 + 3) & ~3) + ((l3 + 3) & ~3) + nw * 64;
+}
+
+// The same iteration driven by a record instead of the tree: body_a over the recorded lists,
+// mid(), body_b over them again.  `at` walks the tile's record stream of `used` words; `lost`
+// is set when the stream does not hold the items this iteration expects (the caller stops).
+template <typename BodyA, typename Mid, typename BodyB>
+__device__ __forceinline__ bool slab_replay(const MarchParams &P, const uint32_t *reg, int used, int &at, bool &lost,
+                                            const RayState &R, bool need, int &p0, float &found, float &searched_to, BodyA body_a,
+                                            Mid mid, BodyB body_b)
+{
+    const int start = at;
+    int end = at; // one past the iteration's last LISTS item
+    while (end + 8 <= used && (uni_u32(reg[end]) & 0xff000000u) == RGX_REC_LISTS && end + lists_size(reg + end) <= used)
+        end += lists_size(reg + end);
+    const uint32_t tr = end + 4 <= used ? uni_u32(reg[end]) : 0u;
+    const bool any_search = tr & 1u;
+    if ((tr & 0xff000000u) != RGX_REC_TRAIL || end + 4 + (any_search ? 64 : 0) > used) {
+        lost = true;
+        mid();
+        return false;
+    }
+    for (int a = start; a < end;) a += replay_lists<true>(P, reg + a, need, p0, body_a);
+    const float cover = __uint_as_float(uni_u32(reg[end + 1]));
+    found = any_search ? __uint_as_float(reg[end + 4 + threadIdx.x]) : -1.0f;
+    searched_to = fminf(R.texit, cover);
+    at = end + 4 + (any_search ? 64 : 0);
+    const bool run = mid();
+    if (__any(run)) {
+        int dummy = 0;
+        for (int b = start; b < end;) b += replay_lists<false>(P, reg + b, run, dummy, body_b);
     }
     return run;
 }
@@ -746,8 +920,9 @@ __device__ __forceinline__ void lane_pixel(int px0, int py0, int &px, int &py)
 __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchParams P)
 {
     RGX_TILE_LDS();
-    int px0, py0;
-    if (!tile_origin(P, px0, py0)) return; // whole wave
+    int px0, py0, tile;
+    if (!tile_origin(P, px0, py0, &tile)) return; // whole wave
+    Recorder rec = {P.records ? P.records + (int64_t)tile * P.rec_tile_words : nullptr, 4, P.rec_tile_words, false, 4};
     int px, py;
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
@@ -772,11 +947,13 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
 #pragma unroll
             for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
             f3 rdt = dir * fmaf(dt, 0.5f, R.tbuffer); // samples 0..15
-            auto accumulate = [&](const float4 *e, bool hit, bool) {
+            auto accumulate = [&](const auto &e, bool hit, bool) {
                 if (hit) {
-                    const Prim *pr = P.prims + __float_as_int(e[4].w);
-                    const float4 col = pr->rgba4;
-                    HitSetup hs = hit_setup(e, pr->pos4, dir, rdt, dt);
+                    const float4 col = e.prim->rgba4;
+                    f3 U, V, W, inv;
+                    float k;
+                    e.frame(U, V, W, inv, k);
+                    HitSetup hs = hit_setup(U, V, W, inv, k, e.prim->pos4, dir, rdt, dt);
                     const float rho = col.w;
 #pragma unroll
                     for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
@@ -812,8 +989,8 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
                 rdt = dir * fmaf(dt, 16.5f, R.tbuffer);
                 return has && R.T > P.m.t_eps;
             };
-            const bool run2 = slab_tables(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, accumulate, second_half,
-                                          accumulate);
+            const bool run2 = slab_tables(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, accumulate,
+                                          second_half, accumulate);
             if (run2) blend();
             if (need && p0 > 0) {
                 cn.slabs++;
@@ -830,6 +1007,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
         P.ray_colors[3 * ray + 1] = Cg + R.T * bg;
         P.ray_colors[3 * ray + 2] = Cb + R.T * bg;
     }
+    rec.finish();
     flush_stats(P.stats, cn);
 }
 
@@ -861,20 +1039,26 @@ __device__ __forceinline__ float row_sum(float v)
 // nineteen running sums; the `power < k^2` mask follows the reference's 32-step
 // recurrence exactly.  The 14 gradient words of a Gaussian are summed over the 16
 // rays of a row with DPP adds before one lane per row adds them to memory.
+template <bool REPLAY>
 __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchParams P)
 {
-    RGX_TILE_LDS();
-    int px0, py0;
-    if (!tile_origin(P, px0, py0)) return; // whole wave
+    int px0, py0, tile;
+    if (!tile_origin(P, px0, py0, &tile)) return; // whole wave
+    const uint32_t *reg = P.records ? P.records + (int64_t)tile * P.rec_tile_words : nullptr;
+    if (REPLAY) {
+        if (uni_u32(reg[0]) != 0u) return; // this tile's record overflowed: the other kernel handles it
+    } else if (P.only_overflow) {
+        if (uni_u32(reg[0]) == 0u) return; // replayed
+    }
     const int lane = threadIdx.x;
     int px, py;
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
     Counters cn;
-    Frustum F;
-    frustum_planes(P.cam, px0, py0, F);
     RayState R;
-    ray_begin<true>(P, px, py, valid, R);
+    // a replay follows the forward's iteration sequence, so it takes the forward's conventions
+    // (reciprocal multiply in the bbox test, clipped slab bounds)
+    ray_begin<!REPLAY>(P, px, py, valid, R);
     const f3 dir = R.dir;
     f3 g = mk3(0.f, 0.f, 0.f);
     float D = 0.f;
@@ -883,11 +1067,11 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
         g = mk3(P.dloss[3 * ray], P.dloss[3 * ray + 1], P.dloss[3 * ray + 2]);
         D = dot3(g, mk3(P.fwd_colors[3 * ray], P.fwd_colors[3 * ray + 1], P.fwd_colors[3 * ray + 2]));
     }
-    Window Wn = {0.f, 0, false, 4};
 
-    while (__any(R.active)) {
+    // one slab iteration; `drive(need, tlo, thi, p0, ov, found, searched_to, body_a, mid, body_b)` supplies the hit lists
+    auto iteration = [&](auto drive) {
         float tlo, thi;
-        const bool need = slab_begin<false>(P, R, tlo, thi);
+        const bool need = slab_begin<REPLAY>(P, R, tlo, thi);
         int p0 = 0;
         bool ov = false;
         float found = -1.0f, searched_to = 0.f;
@@ -899,13 +1083,15 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
             for (int i = 0; i < RGX_BUFFER_SIZE; ++i) PA[i] = PB[i] = 0.f;
             const f3 rdt0 = dir * fmaf(dt, 0.5f, tbuffer);
             const f3 rdt1 = dir * fmaf(dt, 16.5f, tbuffer);
-            auto densities = [&](const float4 *e, bool hit, bool) {
+            auto densities = [&](const auto &e, bool hit, bool) {
                 if (hit) {
-                    const Prim *pr = P.prims + __float_as_int(e[4].w);
-                    const float4 col = pr->rgba4, pos4 = pr->pos4;
+                    const float4 col = e.prim->rgba4, pos4 = e.prim->pos4;
                     const float rho = col.w;
                     const float ddc = dot3(g, mk3(col.x, col.y, col.z));
-                    HitSetup hs = hit_setup(e, pos4, dir, rdt0, dt);
+                    f3 U, V, W, inv;
+                    float k;
+                    e.frame(U, V, W, inv, k);
+                    HitSetup hs = hit_setup(U, V, W, inv, k, pos4, dir, rdt0, dt);
 #pragma unroll
                     for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
                         const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
@@ -914,7 +1100,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
                         hs.power += hs.inc;
                         hs.inc += hs.inc_st;
                     }
-                    hs = hit_setup(e, pos4, dir, rdt1, dt);
+                    hs = hit_setup(U, V, W, inv, k, pos4, dir, rdt1, dt);
 #pragma unroll
                     for (int i = RGX_CHUNK_SIZE; i < RGX_BUFFER_SIZE; ++i) {
                         const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
@@ -952,18 +1138,19 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
             };
             // (3) per table entry: moments per lane, row sum, one set of atomics per row
             const f3 xdir_c = dir * fmaf(dt, 16.0f, tbuffer); // slab centre: t_c = tbuffer + 16 dt
-            auto gradients = [&](const float4 *e, bool hit, bool live) {
+            auto gradients = [&](const auto &e, bool hit, bool live) {
                 float out[14];
 #pragma unroll
                 for (int c = 0; c < 14; ++c) out[c] = 0.f;
-                const int32_t pid = __float_as_int(e[4].w);
+                const int32_t pid = e.pid;
                 if (hit) {
-                    const Prim *pr = P.prims + pid;
-                    const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3], col = pr->rgba4, e5 = pr->pos4;
-                    const float k = e2.w;
-                    const f3 inv_s = mk3(e3.x * k, e3.y * k, e3.z * k);
+                    const Prim *pr = e.prim;
+                    const float4 col = pr->rgba4, e5 = pr->pos4;
+                    f3 U, V, W, inv;
+                    float k;
+                    e.frame(U, V, W, inv, k);
+                    const f3 inv_s = mk3(inv.x * k, inv.y * k, inv.z * k);
                     const float cut = k * k;
-                    const f3 U = mk3(e0.x, e0.y, e0.z), V = mk3(e1.x, e1.y, e1.z), W = mk3(e2.x, e2.y, e2.z);
                     const float rho = col.w;
                     const float dcg = dot3(mk3(col.x, col.y, col.z), g) / rho;
                     // mask recurrence exactly as backward/gaussians_aabb.cu:375-396, 437-438
@@ -1030,7 +1217,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
                     for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, out[c]);
                 }
             };
-            const bool has = slab_tables(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, densities, prefix, gradients);
+            const bool has = drive(need, tlo, thi, p0, ov, found, searched_to, densities, prefix, gradients);
             if (has) {
                 D = D_after;
                 R.T = T_after;
@@ -1040,6 +1227,28 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
             if (ov) cn.overflow++;
         }
         slab_end(R, need, p0, found, searched_to, cn);
+    };
+
+    if constexpr (REPLAY) {
+        const int used = min((int)uni_u32(reg[1]), P.rec_tile_words);
+        int at = 4;
+        bool lost = false;
+        while (__any(R.active) && !lost) {
+            iteration([&](bool need, float, float, int &p0, bool &, float &found, float &searched_to, auto a, auto mid, auto b) {
+                return slab_replay(P, reg, used, at, lost, R, need, p0, found, searched_to, a, mid, b);
+            });
+        }
+        if ((lost || at != used) && lane == 0) cn.replay_lost = 1;
+    } else {
+        RGX_TILE_LDS();
+        Frustum F;
+        frustum_planes(P.cam, px0, py0, F);
+        Window Wn = {0.f, 0, false, 4};
+        Recorder rec = {nullptr, 4, 0, false, 4};
+        while (__any(R.active)) {
+            iteration([&](bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to, auto a, auto mid,
+                          auto b) { return slab_tables(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, a, mid, b); });
+        }
     }
     flush_stats(P.stats, cn);
 }
@@ -1078,10 +1287,11 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
         float found = -1.0f, searched_to = 0.f;
         MarchParams Pc = P;
         Pc.m.max_prim_slice = cap;
-        auto record = [&](const float4 *e, bool hit, bool) {
-            if (hit) ids[ray * cap + written++] = (int32_t)P.order[__float_as_int(e[4].w)];
+        auto record = [&](const auto &e, bool hit, bool) {
+            if (hit) ids[ray * cap + written++] = (int32_t)P.order[e.pid];
         };
-        slab_tables(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, record, [] { return false; }, record);
+        Recorder rec = {nullptr, 4, 0, false, 4};
+        slab_tables(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, record, [] { return false; }, record);
     }
     if (valid) counts[ray] = ov ? -p0 : p0;
 }
@@ -1184,6 +1394,29 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     P.stats = stats;
     P.tiles_x = (cam->width + 7) / 8;
     P.tiles_y = (cam->height + 7) / 8;
+    P.records = nullptr;
+    P.rec_tile_words = 0;
+    P.only_overflow = 0;
+    return RGX_OK;
+}
+
+#define RGX_REC_MIN_TILE_WORDS 1024
+
+extern "C" int rgx_march_records_bytes(int32_t width, int32_t height, int32_t tile_words, size_t *bytes)
+{
+    if (width <= 0 || height <= 0 || tile_words < RGX_REC_MIN_TILE_WORDS || (tile_words & 3) || !bytes) return RGX_EINVAL;
+    *bytes = (size_t)((width + 7) / 8) * (size_t)((height + 7) / 8) * (size_t)tile_words * sizeof(uint32_t);
+    return RGX_OK;
+}
+
+static int attach_records(MarchParams &P, void *records, size_t records_bytes)
+{
+    if (!records) return RGX_OK;
+    const size_t ntiles = (size_t)P.tiles_x * P.tiles_y;
+    const size_t words = records_bytes / sizeof(uint32_t) / ntiles;
+    if (((uintptr_t)records & 15u) || words < RGX_REC_MIN_TILE_WORDS) return RGX_EWORKSPACE;
+    P.records = (uint32_t *)records;
+    P.rec_tile_words = (int32_t)(words > 0x3ffffff ? 0x3ffffff : words) & ~3;
     return RGX_OK;
 }
 
@@ -1194,12 +1427,15 @@ static inline dim3 march_grid(const MarchParams &P)
 }
 
 extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
-                                 float *ray_colors, void *march_ws, size_t march_ws_bytes, RgxStats *stats, void *stream)
+                                 float *ray_colors, void *march_ws, size_t march_ws_bytes, void *records, size_t records_bytes,
+                                 RgxStats *stats, void *stream)
 {
     MarchParams P;
-    const int rc = fill_params(P, ws, cam, march, prims, n, march_ws, march_ws_bytes, stats);
+    int rc = fill_params(P, ws, cam, march, prims, n, march_ws, march_ws_bytes, stats);
     if (rc) return rc;
     if (!ray_colors) return RGX_EINVAL;
+    rc = attach_records(P, records, records_bytes);
+    if (rc) return rc;
     P.ray_colors = ray_colors;
     void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
     hipLaunchKernelGGL(k_march_fwd, march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
@@ -1210,20 +1446,27 @@ extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const Rgx
 
 extern "C" int rgx_march_backward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
                                   const float *ray_colors, const float *dloss, float *ddens, float *drgb, float *dpos,
-                                  float *dscale, float *dquat, void *march_ws, size_t march_ws_bytes, RgxStats *stats,
-                                  void *stream)
+                                  float *dscale, float *dquat, void *march_ws, size_t march_ws_bytes, const void *records,
+                                  size_t records_bytes, RgxStats *stats, void *stream)
 {
     MarchParams P;
-    const int rc = fill_params(P, ws, cam, march, prims, n, march_ws, march_ws_bytes, stats);
+    int rc = fill_params(P, ws, cam, march, prims, n, march_ws, march_ws_bytes, stats);
     if (rc) return rc;
     if (!ray_colors || !dloss || (n > 0 && (!ddens || !drgb || !dpos || !dscale || !dquat))) return RGX_EINVAL;
+    rc = attach_records(P, (void *)records, records_bytes);
+    if (rc) return rc;
     if (n == 0) return RGX_OK;
     P.fwd_colors = ray_colors;
     P.dloss = dloss;
     hipStream_t s = (hipStream_t)stream;
     hipLaunchKernelGGL(k_zero4, grid_for(4 * n, 256), dim3(256), 0, s, (float4 *)P.gbuf, 4 * n);
     void *span = rgx_span_begin(RGX_T_MARCH_BWD, s);
-    hipLaunchKernelGGL(k_march_bwd, march_grid(P), dim3(64), 0, s, P);
+    if (P.records) {
+        // tiles with a complete record replay it; the few whose record overflowed are recomputed
+        hipLaunchKernelGGL(k_march_bwd<true>, march_grid(P), dim3(64), 0, s, P);
+        P.only_overflow = 1;
+    }
+    hipLaunchKernelGGL(k_march_bwd<false>, march_grid(P), dim3(64), 0, s, P);
     rgx_span_end(span, s);
     span = rgx_span_begin(RGX_T_UNPERMUTE, s);
     hipLaunchKernelGGL(k_unpermute_grads, grid_for(n, 256), dim3(256), 0, s, (const float4 *)P.gbuf, P.order, n, ddens, drgb,

@@ -183,21 +183,32 @@ def _march_ws(n, n_rays, max_prim_slice, device):
     return _workspace("march", nbytes, device)
 
 
+REC_TILE_WORDS = 16384   # 64 KiB of hit-list record per 8x8 pixel tile
+
+
+def new_records(cam, device, tile_words=REC_TILE_WORDS):
+    """Buffer for the hit-list record of one forward launch (see rgx_march_records_bytes)."""
+    nbytes = L.size_query(L.lib().rgx_march_records_bytes, C.c_int32(cam.width), C.c_int32(cam.height),
+                          C.c_int32(tile_words))
+    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+
+
 def march_forward(gas, cam, prims, dt_step, dynamic_sampling, max_prim_slice, white_background,
-                  t_eps=TRANSMITTANCE_EPSILON, stats=None):
+                  t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None):
     n, dev = prims.shape[0], prims.device
     n_rays = cam.width * cam.height
     m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), int(bool(white_background)), t_eps)
     ws = _march_ws(n, n_rays, max_prim_slice, dev)
     ray_colors = torch.empty(n_rays, 3, dtype=torch.float32, device=dev)
     L.check(L.lib().rgx_march_forward(L.ptr(gas.ws), C.byref(cam), C.byref(m), L.ptr(prims), C.c_int64(n),
-                                      L.ptr(ray_colors), L.ptr(ws), C.c_size_t(ws.numel()), L.ptr(stats),
+                                      L.ptr(ray_colors), L.ptr(ws), C.c_size_t(ws.numel()), L.ptr(records),
+                                      C.c_size_t(0 if records is None else records.numel()), L.ptr(stats),
                                       L.stream(dev)))
     return ray_colors
 
 
 def march_backward(gas, cam, prims, ray_colors, dloss, dt_step, dynamic_sampling, max_prim_slice,
-                   white_background=True, t_eps=TRANSMITTANCE_EPSILON, stats=None):
+                   white_background=True, t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None):
     n, dev = prims.shape[0], prims.device
     n_rays = cam.width * cam.height
     m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), int(bool(white_background)), t_eps)
@@ -210,6 +221,7 @@ def march_backward(gas, cam, prims, ray_colors, dloss, dt_step, dynamic_sampling
     L.check(L.lib().rgx_march_backward(L.ptr(gas.ws), C.byref(cam), C.byref(m), L.ptr(prims), C.c_int64(n),
                                        L.ptr(ray_colors), L.ptr(dloss), L.ptr(ddens), L.ptr(drgb), L.ptr(dpos),
                                        L.ptr(dscale), L.ptr(dquat), L.ptr(ws), C.c_size_t(ws.numel()),
+                                       L.ptr(records), C.c_size_t(0 if records is None else records.numel()),
                                        L.ptr(stats), L.stream(dev)))
     return ddens, drgb, dpos, dscale, dquat
 

@@ -83,6 +83,8 @@ class RenderOptixSettings:
         self.hit_prim_idx = hit_prim_idx
         self.t_eps = t_eps
         self.stats = None   # optional optix_utils.new_stats() block
+        self.record_hits = True   # forward records its hit lists for the backward to replay
+        self.rec_tile_words = u_ox.REC_TILE_WORDS   # record size per 8x8 pixel tile, 32-bit words
 
 
 def default_settings(viewpoint_cam, dt_step, dynamic_sampling, max_prim_slice, num_sph_gauss=0,
@@ -113,9 +115,12 @@ class RenderOptixFunction(torch.autograd.Function):
         rgb = compute_rgb(cam.eye, positions, color_features, sph_gauss_features, bandwidth_sharpness, lobe_axis,
                           settings.num_sph_gauss, order_sh)
         prims = u_ox.pack_prims(gas, cam, positions, scales, normalized_quaternions, densities, rgb)
+        # when a backward will follow, the forward leaves a record of its hit lists for it to replay
+        records = u_ox.new_records(cam, dev, settings.rec_tile_words) if (any(ctx.needs_input_grad[:8]) and settings.record_hits) else None
         ray_colors = u_ox.march_forward(gas, cam, prims, settings.dt_step, settings.dynamic_sampling,
                                         settings.max_prim_slice, settings.white_background, settings.t_eps,
-                                        settings.stats)
+                                        settings.stats, records)
+        ctx.records = records
         ctx.settings = settings
         ctx.cam = cam
         ctx.gas = gas
@@ -134,7 +139,8 @@ class RenderOptixFunction(torch.autograd.Function):
             densities_grad, rgb_grad, positions_grad, scales_grad, quaternions_grad = u_ox.march_backward(
                 ctx.gas, ctx.cam, ctx.prims, ray_colors, dloss_dray_colors, settings.dt_step,
                 settings.dynamic_sampling, settings.max_prim_slice, settings.white_background, settings.t_eps,
-                settings.stats)
+                settings.stats, ctx.records)
+            ctx.records = None
             sh_grad, dpos_dir, dsg, dsharp, daxis = compute_sh_grad(
                 ctx.cam.eye, positions, color_features, sph_gauss_features, bandwidth_sharpness, lobe_axis,
                 settings.num_sph_gauss, ctx.order_sh, rgb_grad)

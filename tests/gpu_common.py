@@ -19,8 +19,11 @@ def cos_rel(a, b):
     return a @ b / (np.linalg.norm(a) * np.linalg.norm(b) + 1e-300), np.linalg.norm(a - b) / (np.linalg.norm(b) + 1e-300)
 
 
-def gpu_render(scene_np, cam, cfg, white=True, supersampling=(1, 1), want_grad=None, stats=True):
-    """Runs RenderOptixFunction (and its backward when ``want_grad`` = dL/dimage is given)."""
+def gpu_render(scene_np, cam, cfg, white=True, supersampling=(1, 1), want_grad=None, stats=True, record_hits=True,
+               rec_tile_words=None):
+    """Runs RenderOptixFunction (and its backward when ``want_grad`` = dL/dimage is given).
+    ``record_hits``: the backward replays the forward's hit-list record (the default) or searches
+    the tree again; ``rec_tile_words`` sizes the record per tile."""
     sc = to_dev(scene_np)
     names = ("positions", "scales", "quaternions", "densities", "color_features", "sph_gauss_features",
              "bandwidth_sharpness", "lobe_axis")
@@ -34,6 +37,9 @@ def gpu_render(scene_np, cam, cfg, white=True, supersampling=(1, 1), want_grad=N
     settings = default_settings(cam.to(DEV), cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
                                 num_sph_gauss=g, white_background=white, supersampling=supersampling,
                                 t_eps=cfg.get("t_eps", 1e-3))
+    settings.record_hits = record_hits
+    if rec_tile_words is not None:
+        settings.rec_tile_words = rec_tile_words
     if stats:
         settings.stats = u_ox.new_stats(DEV)
     img = RenderOptixFunction.apply(*args, settings)
@@ -47,5 +53,6 @@ def gpu_render(scene_np, cam, cfg, white=True, supersampling=(1, 1), want_grad=N
         out["grads"] = {k: (None if a.grad is None else a.grad.cpu().numpy()) for k, a in zip(names, args)}
         if stats:
             out["stats_bwd"] = u_ox.read_stats(settings.stats)
+            assert out["stats_bwd"]["replay_lost"] == 0
     torch.cuda.synchronize()
     return out

@@ -236,6 +236,36 @@ def test_backward_config0_gradients(gx, orc, c0):
         assert out["grads"][k] is None
 
 
+def test_backward_replay_of_recorded_hit_lists_equals_recomputation(gx, orc):
+    """The backward fed with the forward's hit-list record must give what the backward that
+    searches the tree again gives (same hits, same order; only the atomic summation order may
+    differ), also when some tiles' records overflow and fall back to recomputation, and with
+    the adaptive step and candidate sets that need several table batches."""
+    for label, config, scale, dyn, words in (("fixed step", 0, 3.0, False, None), ("adaptive step", 2, 3.0, True, None),
+                                             ("fat Gaussians, small records", 0, 8.0, False, 1024)):
+        sc = scenes.scene_to_numpy(scenes.make_scene(config, n=5000, sh_degree=1, seed=21))
+        sc["scales"] = sc["scales"] * scale
+        cam = scenes.make_camera(config, 1, width=52, height=44)
+        cfg = dict(dt_step=0.004, dynamic_sampling=dyn, max_prim_slice=4096)
+        dloss = np.random.default_rng(3).normal(size=(52 * 44, 3)).astype(np.float32)
+        _step("replay vs recompute: " + label)
+        a = gx.gpu_render(sc, cam, cfg, want_grad=dloss, record_hits=False)
+        b = gx.gpu_render(sc, cam, cfg, want_grad=dloss, record_hits=True, rec_tile_words=words)
+        assert np.array_equal(a["image"], b["image"])
+        for k in ("hit_pairs", "slabs", "empty_slabs", "overflow_rays", "rays_hit"):
+            assert a["stats_fwd"][k] == b["stats_fwd"][k], k
+        assert a["stats_bwd"]["hit_pairs"] == b["stats_bwd"]["hit_pairs"] > 10000
+        assert a["stats_bwd"]["slabs"] == b["stats_bwd"]["slabs"]
+        if words is None:   # everything replayed: the backward fetched no tree node
+            assert b["stats_bwd"]["nodes_visited"] == 0
+        else:               # some tiles replayed, some recomputed
+            print("nodes", b["stats_bwd"]["nodes_visited"], a["stats_bwd"]["nodes_visited"], flush=True)
+            assert 0 < b["stats_bwd"]["nodes_visited"] <= a["stats_bwd"]["nodes_visited"]
+        for k in ("positions", "scales", "quaternions", "densities", "color_features"):
+            cos, rel = gx.cos_rel(b["grads"][k], a["grads"][k])
+            assert cos >= 1 - 1e-9 and rel <= 2e-5, (label, k, cos, rel)
+
+
 def test_dynamic_sampling_lobes_supersampling_black_background(gx, orc):
     """The unbounded-scene settings (adaptive step, camera inside the cloud) with spherical-Gaussian
     lobes, a non-multiple-of-8 image, 2x1 supersampling and a black background."""

@@ -647,9 +647,7 @@ __device__ __forceinline__ void shade_rows(const MarchParams &P, const TileLds &
 // Hit-list records.  What the filter produces for a slab iteration -- per 4x4 row the Gaussians
 // some ray of the row hits, per ray its hit bits over that list, per searching ray the first-hit
 // t -- is a few hundred bytes.  The forward can stream it to memory so that the backward replays
-// the same lists instead of sweeping the tree and evaluating the predicate again; within one
-// kernel the same records let the second pass of an iteration whose candidates did not fit one
-// table skip its second sweep.  Per tile a region of rec_tile_words 32-bit words:
+// the same lists instead of sweeping the tree and evaluating the predicate again.  Per tile a region of rec_tile_words 32-bit words:
 //   word 0: 0 = complete, 1 = the region overflowed (record unusable);  word 1: words used;
 //   from word 4, per iteration:  one LISTS item per table batch, then a TRAIL item
 //   LISTS: {tag | last << 8 | nw, len[4], -, -, -}, pid[pad4(len[r])] for r = 0..3, mask[nw][64]
@@ -662,7 +660,6 @@ struct Recorder {
     int off;        // next free word (wave-uniform)
     int cap;        // words in the region
     bool ovf;       // the region is exhausted
-    int iter_start; // first item of the current iteration
     __device__ __forceinline__ bool on() const { return reg != nullptr && !ovf; }
 
     __device__ __forceinline__ void write_lists(const TileLds &L, int len, bool last)
@@ -710,6 +707,13 @@ struct Recorder {
             reg[1] = (uint32_t)off;
         }
     }
+};
+
+// Stand-in where nothing is recorded.
+struct NoRecorder {
+    __device__ __forceinline__ void write_lists(const TileLds &, int, bool) {}
+    __device__ __forceinline__ void write_trailer(bool, float, float) {}
+    __device__ __forceinline__ void finish() {}
 };
 
 __device__ __forceinline__ uint32_t uni_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
@@ -766,28 +770,17 @@ __device__ __forceinline__ void frustum_range(Frustum &F, float t0, float t1)
 //   phase 1  body_b over the same row lists, or over freshly swept and filtered batches when the
 //            candidates did not fit one table.
 // Returns the phase-1 participation flag of this lane.
-template <typename BodyA, typename Mid, typename BodyB>
+template <typename Rec, typename BodyA, typename Mid, typename BodyB>
 __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds &L, Frustum &F, Window &Wn, const RayState &R,
                                             bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to,
-                                            Counters &cn, Recorder &rec, BodyA body_a, Mid mid, BodyB body_b)
+                                            Counters &cn, Rec &rec, BodyA body_a, Mid mid, BodyB body_b)
 {
     const bool srch = R.active && R.searching, want = need || srch;
-    rec.iter_start = rec.off;
     const float t0 = wave_min_all(want ? tlo : INFINITY), t1 = wave_max_all(want ? thi : -INFINITY);
     const bool any_search = __any(srch);
     int len = 0, q0 = 0;
     bool run = need, qov = false;
     for (int phase = 0; phase < 2; ++phase) {
-        if (phase == 1 && !Wn.resident && rec.on()) {
-            // the batches of this iteration were recorded: replay them instead of sweeping again
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            __syncthreads();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-            int at = rec.iter_start, dummy = 0;
-            while (at < rec.off && (uni_u32(rec.reg[at]) & 0xff000000u) == RGX_REC_LISTS)
-                at += replay_lists<false>(P, rec.reg + at, run, dummy, body_b);
-            break;
-        }
         const bool reuse = Wn.resident && t1 <= Wn.hi;
         Sweep S = {0};
         if (!reuse) {
@@ -917,12 +910,14 @@ __device__ __forceinline__ void lane_pixel(int px0, int py0, int &px, int &py)
 // ---------------------------------------------------------------------------
 // Forward: __raygen__rg (gaussians_aabb.cu:205-340), accumulateChunk (112-180),
 // colorBlendingT_chunked (182-203).
+template <bool RECORD>
 __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchParams P)
 {
     RGX_TILE_LDS();
     int px0, py0, tile;
     if (!tile_origin(P, px0, py0, &tile)) return; // whole wave
-    Recorder rec = {P.records ? P.records + (int64_t)tile * P.rec_tile_words : nullptr, 4, P.rec_tile_words, false, 4};
+    typename std::conditional<RECORD, Recorder, NoRecorder>::type rec;
+    if constexpr (RECORD) rec = Recorder{P.records + (int64_t)tile * P.rec_tile_words, 4, P.rec_tile_words, false};
     int px, py;
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
@@ -1244,7 +1239,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
         Frustum F;
         frustum_planes(P.cam, px0, py0, F);
         Window Wn = {0.f, 0, false, 4};
-        Recorder rec = {nullptr, 4, 0, false, 4};
+        NoRecorder rec;
         while (__any(R.active)) {
             iteration([&](bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to, auto a, auto mid,
                           auto b) { return slab_tables(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, a, mid, b); });
@@ -1290,7 +1285,7 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
         auto record = [&](const auto &e, bool hit, bool) {
             if (hit) ids[ray * cap + written++] = (int32_t)P.order[e.pid];
         };
-        Recorder rec = {nullptr, 4, 0, false, 4};
+        NoRecorder rec;
         slab_tables(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, record, [] { return false; }, record);
     }
     if (valid) counts[ray] = ov ? -p0 : p0;
@@ -1438,7 +1433,8 @@ extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const Rgx
     if (rc) return rc;
     P.ray_colors = ray_colors;
     void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
-    hipLaunchKernelGGL(k_march_fwd, march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    if (P.records) hipLaunchKernelGGL(k_march_fwd<true>, march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    else hipLaunchKernelGGL(k_march_fwd<false>, march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     rgx_span_end(span, (hipStream_t)stream);
     RGX_LAUNCH_CHECK();
     return RGX_OK;

@@ -178,6 +178,47 @@ def test_forward_config0_image_and_hit_sets(gx, orc, c0):
         assert sorted(ids[s, :cnt[s]].tolist()) == want[s], s
 
 
+def test_config0_against_committed_golden_vectors(gx, orc, c0):
+    """The same configuration-0 results the oracle produced when tests/golden/config0.npz was
+    written: image, march counters, gradients, per-slab hit sets and first-hit distances."""
+    import os
+    import sys
+    from raygaussx_amd import optix_utils as u_ox
+    from raygaussx_amd.render_optix import compute_rgb
+    here = os.path.dirname(os.path.abspath(__file__))
+    sys.path.insert(0, os.path.join(here, "golden"))
+    import make_golden
+    g = np.load(os.path.join(here, "golden", "config0.npz"))
+    _, cam, cfg = c0
+    sc = make_golden.scene_of(g)
+    _step("golden: forward + backward config0")
+    out = gx.gpu_render(sc, cam, cfg, want_grad=make_golden.mse_dloss(g["image"]))
+    assert np.abs(out["image"] - g["image"]).max() <= IMG_TOL
+    for k in ("hit_pairs", "slabs", "empty_slabs", "rays_hit"):
+        assert out["stats_fwd"][k] == int(g["stats_" + k]), k
+    _check_grads(gx, out["grads"], {k[2:]: g[k] for k in g.files if k.startswith("d_")})
+    # the two ray queries on the stored segments
+    d = gx.to_dev(sc)
+    eye = cam.camera_center.numpy()
+    gas = out["settings"].gas
+    rgb = compute_rgb(cam.camera_center, d["positions"], d["color_features"], None, None, None, 0, 3)
+    ps = u_ox.pack_prims(gas, eye, d["positions"], d["scales"], d["quaternions"], d["densities"], rgb)
+
+    def dirs_of(rays):   # computeRay on the host (fp32, no contraction), as the kernels evaluate it
+        return orc.ray_dirs(orc.camera_struct(cam), rays)
+    _step("golden: hit sets")
+    dv = lambda a, t=torch.float32: torch.from_numpy(np.ascontiguousarray(a)).to(gx.DEV, t)
+    cnt, ids = u_ox.trace_segments(gas, ps, eye, dv(dirs_of(g["seg_ray"])), dv(g["seg_lo"]), dv(g["seg_hi"]), 64)
+    cnt, ids = cnt.cpu().numpy(), ids.cpu().numpy()
+    off = g["seg_off"]
+    np.testing.assert_array_equal(cnt, np.diff(off))
+    for s in range(len(cnt)):
+        assert sorted(ids[s, :cnt[s]].tolist()) == g["seg_ids"][off[s]:off[s + 1]].tolist(), s
+    _step("golden: first hits")
+    t = u_ox.first_hit(gas, ps, eye, dv(dirs_of(g["fh_ray"])), dv(g["fh_lo"]), dv(g["fh_hi"])).cpu().numpy()
+    np.testing.assert_array_equal(t, g["fh_t"])
+
+
 def test_tile_cooperative_collect_hit_sets_bit_exact(gx, orc, c0):
     """The collect query as the march kernels run it (one 8x8 tile per wavefront, shared candidate
     gather, per-ray exact predicate) on the oracle's own slab intervals: identical hit sets."""

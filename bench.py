@@ -48,12 +48,15 @@ WORKLOADS = {
     "c4_1M_800x800": (4, 1_000_000, 800, 800),
     "c1_300k_800x800": (1, 300_000, 800, 800),
     "c4_1M_1024x1024": (4, 1_000_000, 1024, 1024),
+    "c2_3M_1237x822": (2, 3_000_000, 1237, 822),
     "c0_4096_128x128": (0, 4096, 128, 128),
+    # inference along a camera path, tree built once (scripts/test.py:60-126): frames per second
+    "c3_3M_1920x1080_fwd": (3, 3_000_000, 1920, 1080),
 }
 
 
-def cpu_baseline(scene, cam, cfg, n_sample, threads):
-    """Forward + backward of the CPU oracle on a strided ray sample of the same view."""
+def cpu_baseline(scene, cam, cfg, n_sample, threads, backward=True):
+    """Forward (+ backward) of the CPU oracle on a strided ray sample of the same view."""
     from oracle import oracle as orc
     orc.build()
     orc.set_num_threads(threads)
@@ -63,11 +66,12 @@ def cpu_baseline(scene, cam, cfg, n_sample, threads):
     t0 = time.perf_counter()
     img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
                                       ray_ids=ids)
-    dloss = np.full(img.shape, 1.0 / img.size, np.float32)
-    orc.render_backward(sc, ctx, img, dloss)
+    if backward:
+        dloss = np.full(img.shape, 1.0 / img.size, np.float32)
+        orc.render_backward(sc, ctx, img, dloss)
     dt = time.perf_counter() - t0
     return dict(value=round(n_sample / dt / 1e6, 6), unit="Mrays/s", cores=threads, kind="port",
-                sample=f"{n_sample} strided rays of camera 0, fwd+bwd, all {sc['positions'].shape[0]} Gaussians "
+                sample=f"{n_sample} strided rays of camera 0, {'fwd+bwd' if backward else 'fwd'}, all {sc['positions'].shape[0]} Gaussians "
                        f"(brute-force hit search), {dt:.1f} s")
 
 
@@ -112,9 +116,21 @@ def main():
     target = torch.rand(n_rays, 3, device=dev, generator=torch.Generator(dev).manual_seed(1))
     stats = u_ox.new_stats(dev)
     gas = None
+    inference = args.workload.endswith("_fwd")
+    if inference:
+        args.forward_only = True
+        from raygaussx_amd.render_optix import compute_rgb
+        tree = u_ox.AccelerationStructure(n, dev).build_from_gaussians(dscene["positions"], dscene["scales"],
+                                                                        dscene["quaternions"], dscene["densities"])
 
     def step(i):
         nonlocal gas
+        if inference:   # per frame: view-dependent colour, primitive records, march
+            cam = cams[(7 * i) % n_cams]
+            rgb = compute_rgb(cam.camera_center, dscene["positions"], dscene["color_features"], None, None, None, 0, 3)
+            return u_ox.launch_pipeline_test(None, None, tree, None, None, cfg["dt_step"], cfg["dynamic_sampling"], cam,
+                                             dscene["densities"], rgb, dscene["positions"], dscene["scales"],
+                                             dscene["quaternions"], cfg["max_prim_slice"], t_eps=cfg["t_eps"], stats=stats)
         s = default_settings(cams[i % n_cams], cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
                              t_eps=cfg["t_eps"], gas=gas)
         s.stats = stats
@@ -167,8 +183,10 @@ def main():
                higher_is_better=True, scaling="weak", vs_baseline=None, dtype="f32", data="synthetic",
                config=dict(workload=args.workload, gaussians=n, width=width, height=height, sh_degree=3,
                            dt_step=cfg["dt_step"], dynamic_sampling=cfg["dynamic_sampling"],
-                           max_prim_slice=cfg["max_prim_slice"], step="bvh build + sh + pack + march fwd"
-                           + ("" if args.forward_only else " + march bwd + sh bwd") + ", 1 view"),
+                           max_prim_slice=cfg["max_prim_slice"], t_eps=cfg["t_eps"],
+                           step=("sh + pack + march fwd, 1 view, tree built once" if inference else
+                                 "bvh build + sh + pack + march fwd"
+                                 + ("" if args.forward_only else " + march bwd + sh bwd") + ", 1 view")),
                roofline=roofline,
                step_roofline=dict(bytes_per_step=int(step_bytes),
                                   achieved=round(step_bytes / (ms_per_step * 1e-3) / 1e9, 2), unit="GB/s",
@@ -176,10 +194,13 @@ def main():
                                   roofline_mrays=round(HBM_PEAK_GBPS * 1e9 * n_rays / step_bytes / 1e6, 2)),
                kernels_ms={k: round(v[0] / max(v[1], 1), 4) for k, v in timing.items() if v[1]},
                stats_per_step={k: v / args.steps for k, v in st.items()})
+    if inference:
+        out["frames_per_s"] = round(1e3 / ms_per_step, 3)
     if args.cpu_rays > 0:
         threads = min(16, os.cpu_count() or 1)
         out["cpu_baseline"] = cpu_baseline(scene, scenes.make_camera(config, 0, width=width, height=height), cfg,
-                                           args.cpu_rays, threads)
+                                           args.cpu_rays if n <= 1_000_000 else min(args.cpu_rays, 4096), threads,
+                                           backward=not args.forward_only)
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out), flush=True)

@@ -643,6 +643,32 @@ __device__ __forceinline__ void shade_rows(const MarchParams &P, const TileLds &
     }
 }
 
+// Shade, one ray at a time: every lane walks its own hits (the set bits of its mask over its
+// row's list), so the trip count is the longest hit list of a ray instead of the longest row list.
+// For bodies that need no sum over the rays of a row.  The order of a ray's hits is that of
+// shade_rows.
+template <typename Body>
+__device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds &L, int len, bool run, Body body)
+{
+    const int lane = threadIdx.x, row = lane >> 4;
+    const int nw = (len + 31) >> 5;
+    int w = 0;
+    uint32_t bits = (run && nw > 0) ? L.mask[0][lane] : 0u;
+    for (;;) {
+        while (bits == 0u && run && w + 1 < nw) bits = L.mask[++w][lane];
+        const bool has = bits != 0u;
+        if (!__any(has)) break;
+        int c = 0;
+        if (has) {
+            c = L.rowlist[row * RGX_CCAP + w * 32 + __builtin_ctz(bits)];
+            bits &= bits - 1u;
+        }
+        const float4 *tab = (const float4 *)(L.tab + c * RGX_TAB);
+        const int32_t pid = __float_as_int(L.tab[c * RGX_TAB + 19]);
+        body(Entry<true>{tab, P.prims + pid, pid}, has, has);
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Hit-list records.  What the filter produces for a slab iteration -- per 4x4 row the Gaussians
 // some ray of the row hits, per ray its hit bits over that list, per searching ray the first-hit
@@ -718,9 +744,10 @@ struct NoRecorder {
 
 __device__ __forceinline__ uint32_t uni_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
-// Replays one LISTS item: the four rows walk their recorded lists in lock step, exactly as
-// shade_rows does on a live table.  COUNT adds the lane's hits to p0.  Returns the item's size.
-template <bool COUNT, typename Body>
+// Replays one LISTS item as shade_rows (the four rows walk their recorded lists in lock step) or,
+// with LANES, as shade_lanes (every ray walks its own hits) does on a live table.  COUNT adds the
+// lane's hits to p0.  Returns the item's size.
+template <bool COUNT, bool LANES, typename Body>
 __device__ __forceinline__ int replay_lists(const MarchParams &P, const uint32_t *it, bool run, int &p0, Body body)
 {
     const int lane = threadIdx.x, row = lane >> 4;
@@ -729,17 +756,36 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const uint32_t
     const int q0 = (l0 + 3) & ~3, q1 = (l1 + 3) & ~3, q2 = (l2 + 3) & ~3, q3 = (l3 + 3) & ~3;
     const int len = row == 0 ? l0 : row == 1 ? l1 : row == 2 ? l2 : l3;
     const uint32_t *pids = it + 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0);
-    const uint32_t *masks = it + 8 + q0 + q1 + q2 + q3;
-    const int maxlen = max(max(l0, l1), max(l2, l3));
-    uint32_t bits = 0;
-    for (int i = 0; i < maxlen; ++i) {
-        if ((i & 31) == 0) bits = masks[(i >> 5) * 64 + lane];
-        const bool live = i < len;
-        const bool hit = run && live && ((bits >> (i & 31)) & 1u);
-        if (COUNT && hit) ++p0;
-        if (__ballot(hit)) {
-            const int32_t pid = live ? (int32_t)pids[i] : 0;
-            body(Entry<false>{nullptr, P.prims + pid, pid}, hit, live);
+    const uint32_t *masks = it + 8 + q0 + q1 + q2 + q3 + lane; // word w of this lane: masks[w * 64]
+    if constexpr (LANES) {
+        const int nwr = run ? (len + 31) >> 5 : 0; // words of this lane's row; later words are not its own
+        if (COUNT)
+            for (int w = 0; w < nwr; ++w) p0 += __popc(masks[w * 64]);
+        int w = 0;
+        uint32_t bits = nwr > 0 ? masks[0] : 0u;
+        for (;;) {
+            while (bits == 0u && w + 1 < nwr) bits = masks[++w * 64];
+            const bool has = bits != 0u;
+            if (!__any(has)) break;
+            int32_t pid = 0;
+            if (has) {
+                pid = (int32_t)pids[w * 32 + __builtin_ctz(bits)];
+                bits &= bits - 1u;
+            }
+            body(Entry<false>{nullptr, P.prims + pid, pid}, has, has);
+        }
+    } else {
+        const int maxlen = max(max(l0, l1), max(l2, l3));
+        uint32_t bits = 0;
+        for (int i = 0; i < maxlen; ++i) {
+            if ((i & 31) == 0) bits = masks[(i >> 5) * 64];
+            const bool live = i < len;
+            const bool hit = run && live && ((bits >> (i & 31)) & 1u);
+            if (COUNT && hit) ++p0;
+            if (__ballot(hit)) {
+                const int32_t pid = live ? (int32_t)pids[i] : 0;
+                body(Entry<false>{nullptr, P.prims + pid, pid}, hit, live);
+            }
         }
     }
     return 8 + q0 + q1 + q2 + q3 + nw * 64;
@@ -769,8 +815,10 @@ __device__ __forceinline__ void frustum_range(Frustum &F, float t0, float t1)
 //   mid()    per lane, between the phases; returns whether the lane takes part in phase 1;
 //   phase 1  body_b over the same row lists, or over freshly swept and filtered batches when the
 //            candidates did not fit one table.
+// LANES_A / LANES_B: the body needs no sums over a row's rays, so every ray walks its own hits
+// (shade_lanes) instead of the rows walking their lists in lock step (shade_rows).
 // Returns the phase-1 participation flag of this lane.
-template <typename Rec, typename BodyA, typename Mid, typename BodyB>
+template <bool LANES_A, bool LANES_B, typename Rec, typename BodyA, typename Mid, typename BodyB>
 __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds &L, Frustum &F, Window &Wn, const RayState &R,
                                             bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to,
                                             Counters &cn, Rec &rec, BodyA body_a, Mid mid, BodyB body_b)
@@ -836,10 +884,14 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                     qov = cut;
                 }
             }
-            if constexpr (std::is_same<BodyA, BodyB>::value) {
-                shade_rows(P, L, len, run, body_a);
+            if constexpr (std::is_same<BodyA, BodyB>::value && LANES_A == LANES_B) {
+                if constexpr (LANES_A) shade_lanes(P, L, len, run, body_a);
+                else shade_rows(P, L, len, run, body_a);
+            } else if (phase == 0) {
+                if constexpr (LANES_A) shade_lanes(P, L, len, run, body_a);
+                else shade_rows(P, L, len, run, body_a);
             } else {
-                if (phase == 0) shade_rows(P, L, len, run, body_a);
+                if constexpr (LANES_B) shade_lanes(P, L, len, run, body_b);
                 else shade_rows(P, L, len, run, body_b);
             }
         }
@@ -863,7 +915,7 @@ __device__ __forceinline__ int lists_size(const uint32_t *it)
 // The same iteration driven by a record instead of the tree: body_a over the recorded lists,
 // mid(), body_b over them again.  `at` walks the tile's record stream of `used` words; `lost`
 // is set when the stream does not hold the items this iteration expects (the caller stops).
-template <typename BodyA, typename Mid, typename BodyB>
+template <bool LANES_A, bool LANES_B, typename BodyA, typename Mid, typename BodyB>
 __device__ __forceinline__ bool slab_replay(const MarchParams &P, const uint32_t *reg, int used, int &at, bool &lost,
                                             const RayState &R, bool need, int &p0, float &found, float &searched_to, BodyA body_a,
                                             Mid mid, BodyB body_b)
@@ -879,7 +931,7 @@ __device__ __forceinline__ bool slab_replay(const MarchParams &P, const uint32_t
         mid();
         return false;
     }
-    for (int a = start; a < end;) a += replay_lists<true>(P, reg + a, need, p0, body_a);
+    for (int a = start; a < end;) a += replay_lists<true, LANES_A>(P, reg + a, need, p0, body_a);
     const float cover = __uint_as_float(uni_u32(reg[end + 1]));
     found = any_search ? __uint_as_float(reg[end + 4 + threadIdx.x]) : -1.0f;
     searched_to = fminf(R.texit, cover);
@@ -887,7 +939,7 @@ __device__ __forceinline__ bool slab_replay(const MarchParams &P, const uint32_t
     const bool run = mid();
     if (__any(run)) {
         int dummy = 0;
-        for (int b = start; b < end;) b += replay_lists<false>(P, reg + b, run, dummy, body_b);
+        for (int b = start; b < end;) b += replay_lists<false, LANES_B>(P, reg + b, run, dummy, body_b);
     }
     return run;
 }
@@ -984,7 +1036,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
                 rdt = dir * fmaf(dt, 16.5f, R.tbuffer);
                 return has && R.T > P.m.t_eps;
             };
-            const bool run2 = slab_tables(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, accumulate,
+            const bool run2 = slab_tables<true, true>(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, accumulate,
                                           second_half, accumulate);
             if (run2) blend();
             if (need && p0 > 0) {
@@ -1230,7 +1282,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
         bool lost = false;
         while (__any(R.active) && !lost) {
             iteration([&](bool need, float, float, int &p0, bool &, float &found, float &searched_to, auto a, auto mid, auto b) {
-                return slab_replay(P, reg, used, at, lost, R, need, p0, found, searched_to, a, mid, b);
+                return slab_replay<true, false>(P, reg, used, at, lost, R, need, p0, found, searched_to, a, mid, b);
             });
         }
         if ((lost || at != used) && lane == 0) cn.replay_lost = 1;
@@ -1242,7 +1294,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
         NoRecorder rec;
         while (__any(R.active)) {
             iteration([&](bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to, auto a, auto mid,
-                          auto b) { return slab_tables(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, a, mid, b); });
+                          auto b) { return slab_tables<true, false>(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, a, mid, b); });
         }
     }
     flush_stats(P.stats, cn);
@@ -1286,7 +1338,7 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
             if (hit) ids[ray * cap + written++] = (int32_t)P.order[e.pid];
         };
         NoRecorder rec;
-        slab_tables(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, record, [] { return false; }, record);
+        slab_tables<false, false>(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, record, [] { return false; }, record);
     }
     if (valid) counts[ray] = ov ? -p0 : p0;
 }

@@ -347,17 +347,39 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
     return C;
 }
 
+// Workgroups are dealt round-robin to the 8 XCDs (workgroup i runs on XCD i % 8), each with its
+// own L2.  The image is cut into blocks of RGX_BLOCK_W x RGX_BLOCK_H tiles and the blocks are
+// dealt to the XCDs in turn: an XCD works through adjacent tiles, so its L2 sees one region of
+// the scene at a time, and every XCD gets blocks from all over the image, so the expensive
+// middle of a scene is not one XCD's alone.  The number of blocks per row of blocks is kept odd
+// (by a phantom block column if need be): with an even count the same few block columns would go
+// to the same XCD in every row.
+#define RGX_BLOCK_W 4
+#define RGX_BLOCK_H 4
+struct TileGrid {
+    int bw, blocks_x, per_xcd; // block width in tiles (clipped to the image), blocks per row of blocks, blocks per XCD
+};
+__host__ __device__ __forceinline__ TileGrid tile_grid(int tiles_x, int tiles_y)
+{
+    TileGrid g;
+    g.bw = tiles_x < RGX_BLOCK_W ? tiles_x : RGX_BLOCK_W;
+    g.blocks_x = ((tiles_x + g.bw - 1) / g.bw) | 1;
+    const int blocks_y = (tiles_y + RGX_BLOCK_H - 1) / RGX_BLOCK_H;
+    g.per_xcd = (g.blocks_x * blocks_y + 7) >> 3;
+    return g;
+}
 __device__ __forceinline__ bool tile_origin(const MarchParams &P, int &px0, int &py0, int *tile_out = nullptr)
 {
-    // Workgroups are dealt round-robin to the 8 XCDs; give each XCD one contiguous
-    // band of tiles so its L2 sees one region of the scene.
-    const int ntiles = P.tiles_x * P.tiles_y;
-    const int per = (gridDim.x + 7) >> 3;
-    const int tile = (blockIdx.x & 7) * per + (blockIdx.x >> 3);
-    px0 = (tile % P.tiles_x) * 8;
-    py0 = (tile / P.tiles_x) * 8;
-    if (tile_out) *tile_out = tile;
-    return tile < ntiles;
+    const TileGrid g = tile_grid(P.tiles_x, P.tiles_y);
+    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int per_block = g.bw * RGX_BLOCK_H;
+    const int block = xcd + 8 * (j / per_block), within = j % per_block;
+    const int tx = (block % g.blocks_x) * g.bw + within % g.bw;
+    const int ty = (block / g.blocks_x) * RGX_BLOCK_H + within / g.bw;
+    px0 = tx * 8;
+    py0 = ty * 8;
+    if (tile_out) *tile_out = ty * P.tiles_x + tx;
+    return tx < P.tiles_x && ty < P.tiles_y;
 }
 
 __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
@@ -479,12 +501,23 @@ __device__ __forceinline__ void slab_end(RayState &R, bool need, int p0, float f
     }
 }
 
+// OR over the 16 lanes of each row, left in every lane of the row
+__device__ __forceinline__ uint32_t row_or(uint32_t v)
+{
+    v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false);  // quad_perm [1,0,3,2]
+    v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false);  // quad_perm [2,3,0,1]
+    v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, false); // row_half_mirror
+    v |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, false); // row_mirror
+    return v;
+}
+
 // ---------------------------------------------------------------------------
 struct TileLds {
     int32_t *queue;        // [RGX_QCAP]
     float *tab;            // [RGX_CCAP * RGX_TAB]
     uint8_t *rowlist;      // [4][RGX_CCAP]: per 16-lane row, table slots some lane of the row hits
     uint32_t (*mask)[64];  // [RGX_CCAP / 32][64]: per lane, hit bits over its row's list
+    uint32_t (*half)[4][RGX_CCAP / 32]; // [2][row][word]: list entries with samples in the slab's first / second 16
 };
 
 // Ray-interval-independent half of __intersection__gaussian (gaussians_aabb.cu:43-82) on a table
@@ -534,6 +567,9 @@ struct Entry {
     }
 };
 
+// exp(-power / 2) as one multiply and the hardware's exp2: -0.5 and log2(e) folded into one constant.
+__device__ __forceinline__ float gauss_weight(float power) { return __builtin_amdgcn_exp2f(power * -0.72134752044448170f); }
+
 // Per-hit constants of the sample recurrence (gaussians_aabb.cu:135-164).
 struct HitSetup {
     float power, inc, inc_st, cut;
@@ -562,12 +598,16 @@ struct LaneQuery {
     bool search;    // searching: smallest hit t in [slo, shi] (the first-hit query, 234-247, 370-380)
     float slo, shi;
     int cap;        // max_prim_slice
+    float tmid;     // tbuffer + 16 dt: where the slab's second 16 samples begin
 };
 
 // Filter: every lane tests the table entries whose distance shell meets [t0, t1] (the union of
 // the lanes' intervals).  A wave is four 16-lane rows, each row a 4x4 pixel block; an entry hit
 // by any marching lane of a row is appended to that row's list, and each lane keeps its own hit
-// bits over its row's list.  len (row-uniform) is the list length; p0 / ov count this lane's
+// bits over its row's list.  Per list entry the row also notes whether any of its rays can have
+// samples inside the Gaussian in the slab's first 16 samples and in its second 16 (the chord
+// [r1, r2] against tmid; a sample lies half a step from tmid, rounding moves a root by far less),
+// so that each half is shaded from its own, shorter list.  len (row-uniform) is the list length; p0 / ov count this lane's
 // hits and note the max_prim_slice cut (__anyhit__ah's optixTerminateRay, 352-356); found is
 // the running minimum of the searching lanes.
 __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, float t1, const LaneQuery &Q, int &p0, bool &ov,
@@ -575,7 +615,16 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
 {
     const int lane = threadIdx.x, row = lane >> 4;
     len = 0;
-    uint32_t bits = 0;
+    uint32_t bits = 0, first = 0, second = 0; // this lane's hits; those with samples in the first / second half
+    auto flush = [&](int w) {
+        L.mask[w][lane] = bits;
+        const uint32_t f = row_or(first), g = row_or(second);
+        if ((lane & 15) == 0) {
+            L.half[0][row][w] = f;
+            L.half[1][row][w] = g;
+        }
+        bits = first = second = 0;
+    };
     for (int h = 0; h < RGX_CCAP / 64; ++h) {
         const int cl = h * 64 + lane;
         bool rel = false;
@@ -590,6 +639,7 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
             m &= m - 1;
             float r1, r2, t;
             bool hit = false;
+            uint32_t in_first = 0, in_second = 0;
             if ((Q.need && !ov) || Q.search) {
                 if (lane_roots((const float4 *)(L.tab + c * RGX_TAB), Q.dir, r1, r2)) {
                     if (Q.search) {
@@ -599,6 +649,8 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
                         else {
                             ++p0;
                             hit = true;
+                            in_first = r1 < Q.tmid ? 1u : 0u;
+                            in_second = r2 > Q.tmid ? 1u : 0u;
                         }
                     }
                 }
@@ -607,18 +659,23 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
             if (lane == 0 && bal) cn.cands_hit++;
             if ((bal >> (row * 16)) & 0xffffull) {
                 bits |= (uint32_t)hit << (len & 31);
+                first |= in_first << (len & 31);
+                second |= in_second << (len & 31);
                 if ((lane & 15) == 0) L.rowlist[row * RGX_CCAP + len] = (uint8_t)c;
                 ++len;
-                if ((len & 31) == 0) {
-                    L.mask[(len >> 5) - 1][lane] = bits;
-                    bits = 0;
-                }
+                if ((len & 31) == 0) flush((len >> 5) - 1);
             }
         }
     }
-    if (len & 31) L.mask[len >> 5][lane] = bits;
+    if (len & 31) flush(len >> 5);
     __syncthreads();
 }
+
+// Tag telling a shading body which 16 of the slab's 32 samples its walk is for.
+template <int H>
+struct Half {
+    static constexpr int value = H;
+};
 
 // Shade: the four rows walk their own lists in lock step; body(entry, hit, live) runs whenever
 // some lane hits (hit: this lane hits this entry; live: this lane's row still has an entry at i).
@@ -638,7 +695,7 @@ __device__ __forceinline__ void shade_rows(const MarchParams &P, const TileLds &
             const int c = live ? L.rowlist[row * RGX_CCAP + i] : 0;
             const float4 *tab = (const float4 *)(L.tab + c * RGX_TAB);
             const int32_t pid = __float_as_int(L.tab[c * RGX_TAB + 19]);
-            body(Entry<true>{tab, P.prims + pid, pid}, hit, live);
+            body(Entry<true>{tab, P.prims + pid, pid}, hit, live, Half<0>{});
         }
     }
 }
@@ -646,16 +703,25 @@ __device__ __forceinline__ void shade_rows(const MarchParams &P, const TileLds &
 // Shade, one ray at a time: every lane walks its own hits (the set bits of its mask over its
 // row's list), so the trip count is the longest hit list of a ray instead of the longest row list.
 // For bodies that need no sum over the rays of a row.  The order of a ray's hits is that of
-// shade_rows.
-template <typename Body>
-__device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds &L, int len, bool run, Body body)
+// shade_rows.  Only the entries that can reach half `half` of the slab's samples are visited; the
+// body gets Half<TAG>.
+#ifdef RGX_NOHALF_WALK
+#define RGX_HALF(x) 0xffffffffu
+#else
+#define RGX_HALF(x) (x)
+#endif
+template <int TAG, typename Body>
+__device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds &L, int len, bool run, int half, Body body)
 {
     const int lane = threadIdx.x, row = lane >> 4;
     const int nw = (len + 31) >> 5;
     int w = 0;
-    uint32_t bits = (run && nw > 0) ? L.mask[0][lane] : 0u;
+    uint32_t bits = (run && nw > 0) ? L.mask[0][lane] & RGX_HALF(L.half[half][row][0]) : 0u;
     for (;;) {
-        while (bits == 0u && run && w + 1 < nw) bits = L.mask[++w][lane];
+        while (bits == 0u && run && w + 1 < nw) {
+            ++w;
+            bits = L.mask[w][lane] & RGX_HALF(L.half[half][row][w]);
+        }
         const bool has = bits != 0u;
         if (!__any(has)) break;
         int c = 0;
@@ -665,7 +731,7 @@ __device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds 
         }
         const float4 *tab = (const float4 *)(L.tab + c * RGX_TAB);
         const int32_t pid = __float_as_int(L.tab[c * RGX_TAB + 19]);
-        body(Entry<true>{tab, P.prims + pid, pid}, has, has);
+        body(Entry<true>{tab, P.prims + pid, pid}, has, has, Half<TAG>{});
     }
 }
 
@@ -676,7 +742,8 @@ __device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds 
 // the same lists instead of sweeping the tree and evaluating the predicate again.  Per tile a region of rec_tile_words 32-bit words:
 //   word 0: 0 = complete, 1 = the region overflowed (record unusable);  word 1: words used;
 //   from word 4, per iteration:  one LISTS item per table batch, then a TRAIL item
-//   LISTS: {tag | last << 8 | nw, len[4], -, -, -}, pid[pad4(len[r])] for r = 0..3, mask[nw][64]
+//   LISTS: {tag | last << 8 | nw, len[4], -, -, -}, pid[pad4(len[r])] for r = 0..3, mask[nw][64],
+//          half[2][4][nw]   (the TileLds arrays of the same names; words past a row's length are junk)
 //   TRAIL: {tag | any_search, cover (float), -, -}, found[64] when any_search
 #define RGX_REC_LISTS 0x4C000000u
 #define RGX_REC_TRAIL 0x54000000u
@@ -696,7 +763,7 @@ struct Recorder {
         const int l2 = __builtin_amdgcn_readlane(len, 32), l3 = __builtin_amdgcn_readlane(len, 48);
         const int nw = (max(max(l0, l1), max(l2, l3)) + 31) >> 5;
         const int p0 = (l0 + 3) & ~3, p1 = (l1 + 3) & ~3, p2 = (l2 + 3) & ~3, p3 = (l3 + 3) & ~3;
-        const int size = 8 + p0 + p1 + p2 + p3 + nw * 64;
+        const int size = 8 + p0 + p1 + p2 + p3 + nw * 72;
         if (off + size + 72 > cap) { // always leave room for the iteration's trailer
             ovf = true;
             return;
@@ -711,6 +778,8 @@ struct Recorder {
             it[base + i] = __float_as_uint(L.tab[L.rowlist[row * RGX_CCAP + i] * RGX_TAB + 19]);
         const int mbase = 8 + p0 + p1 + p2 + p3;
         for (int w = 0; w < nw; ++w) it[mbase + w * 64 + lane] = L.mask[w][lane];
+        if ((lane & 15) < 2) // two lanes per row: one per half
+            for (int w = 0; w < nw; ++w) it[mbase + nw * 64 + ((lane & 15) * 4 + row) * nw + w] = L.half[lane & 15][row][w];
         off += size;
     }
 
@@ -745,9 +814,9 @@ struct NoRecorder {
 __device__ __forceinline__ uint32_t uni_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
 // Replays one LISTS item as shade_rows (the four rows walk their recorded lists in lock step) or,
-// with LANES, as shade_lanes (every ray walks its own hits) does on a live table.  COUNT adds the
-// lane's hits to p0.  Returns the item's size.
-template <bool COUNT, bool LANES, typename Body>
+// with HALF >= 0, as shade_lanes<HALF> (every ray walks its own hits) does on a live table.  COUNT
+// adds the lane's hits to p0.  Returns the item's size.
+template <bool COUNT, int HALF, typename Body>
 __device__ __forceinline__ int replay_lists(const MarchParams &P, const uint32_t *it, bool run, int &p0, Body body)
 {
     const int lane = threadIdx.x, row = lane >> 4;
@@ -757,14 +826,18 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const uint32_t
     const int len = row == 0 ? l0 : row == 1 ? l1 : row == 2 ? l2 : l3;
     const uint32_t *pids = it + 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0);
     const uint32_t *masks = it + 8 + q0 + q1 + q2 + q3 + lane; // word w of this lane: masks[w * 64]
-    if constexpr (LANES) {
+    if constexpr (HALF >= 0) {
         const int nwr = run ? (len + 31) >> 5 : 0; // words of this lane's row; later words are not its own
+        const uint32_t *half = it + 8 + q0 + q1 + q2 + q3 + nw * 64 + (HALF * 4 + row) * nw;
         if (COUNT)
             for (int w = 0; w < nwr; ++w) p0 += __popc(masks[w * 64]);
         int w = 0;
-        uint32_t bits = nwr > 0 ? masks[0] : 0u;
+        uint32_t bits = nwr > 0 ? masks[0] & half[0] : 0u;
         for (;;) {
-            while (bits == 0u && w + 1 < nwr) bits = masks[++w * 64];
+            while (bits == 0u && w + 1 < nwr) {
+                ++w;
+                bits = masks[w * 64] & half[w];
+            }
             const bool has = bits != 0u;
             if (!__any(has)) break;
             int32_t pid = 0;
@@ -772,7 +845,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const uint32_t
                 pid = (int32_t)pids[w * 32 + __builtin_ctz(bits)];
                 bits &= bits - 1u;
             }
-            body(Entry<false>{nullptr, P.prims + pid, pid}, has, has);
+            body(Entry<false>{nullptr, P.prims + pid, pid}, has, has, Half<(HALF < 0 ? 0 : HALF)>{});
         }
     } else {
         const int maxlen = max(max(l0, l1), max(l2, l3));
@@ -784,11 +857,11 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const uint32_t
             if (COUNT && hit) ++p0;
             if (__ballot(hit)) {
                 const int32_t pid = live ? (int32_t)pids[i] : 0;
-                body(Entry<false>{nullptr, P.prims + pid, pid}, hit, live);
+                body(Entry<false>{nullptr, P.prims + pid, pid}, hit, live, Half<0>{});
             }
         }
     }
-    return 8 + q0 + q1 + q2 + q3 + nw * 64;
+    return 8 + q0 + q1 + q2 + q3 + nw * 72;
 }
 
 // Resident candidate window: the table holds every Gaussian of the tile frustum between the
@@ -815,10 +888,12 @@ __device__ __forceinline__ void frustum_range(Frustum &F, float t0, float t1)
 //   mid()    per lane, between the phases; returns whether the lane takes part in phase 1;
 //   phase 1  body_b over the same row lists, or over freshly swept and filtered batches when the
 //            candidates did not fit one table.
-// LANES_A / LANES_B: the body needs no sums over a row's rays, so every ray walks its own hits
-// (shade_lanes) instead of the rows walking their lists in lock step (shade_rows).
+// WALK_FORWARD: body_a per ray over the entries reaching the first 16 samples, body_b per ray over
+// those reaching the second 16.  WALK_BACKWARD: body_a per ray, once for each half; body_b over the
+// row lists in lock step (it sums over the rays of a row).  WALK_ROWS: both bodies over the row lists.
 // Returns the phase-1 participation flag of this lane.
-template <bool LANES_A, bool LANES_B, typename Rec, typename BodyA, typename Mid, typename BodyB>
+enum { WALK_FORWARD, WALK_BACKWARD, WALK_ROWS };
+template <int WALK, typename Rec, typename BodyA, typename Mid, typename BodyB>
 __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds &L, Frustum &F, Window &Wn, const RayState &R,
                                             bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to,
                                             Counters &cn, Rec &rec, BodyA body_a, Mid mid, BodyB body_b)
@@ -868,7 +943,8 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
             if (phase == 0 || !Wn.resident) {
                 // phase 0 asks the lane's real question; a phase-1 re-filter only recounts the slab hits
                 const float cover = Wn.resident ? Wn.hi : t1; // this iteration's tables cover [t0, cover]
-                const LaneQuery Q = {R.dir, run, tlo, thi, phase == 0 && srch, R.tbuffer, fminf(R.texit, cover), P.m.max_prim_slice};
+                const LaneQuery Q = {R.dir, run, tlo, thi, phase == 0 && srch, R.tbuffer, fminf(R.texit, cover), P.m.max_prim_slice,
+                                     fmaf(R.dt, (float)RGX_CHUNK_SIZE, R.tbuffer)};
                 int cnt = phase == 0 ? p0 : q0;
                 bool cut = phase == 0 ? ov : qov;
                 float best = phase == 0 ? found : -1.0f;
@@ -884,14 +960,18 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                     qov = cut;
                 }
             }
-            if constexpr (std::is_same<BodyA, BodyB>::value && LANES_A == LANES_B) {
-                if constexpr (LANES_A) shade_lanes(P, L, len, run, body_a);
-                else shade_rows(P, L, len, run, body_a);
-            } else if (phase == 0) {
-                if constexpr (LANES_A) shade_lanes(P, L, len, run, body_a);
-                else shade_rows(P, L, len, run, body_a);
+            if constexpr (WALK == WALK_FORWARD) {
+                static_assert(std::is_same<BodyA, BodyB>::value, "the forward shades both halves with one body");
+                shade_lanes<0>(P, L, len, run, phase, body_a);
+            } else if constexpr (WALK == WALK_BACKWARD) {
+                if (phase == 0) {
+                    shade_lanes<0>(P, L, len, run, 0, body_a);
+                    shade_lanes<1>(P, L, len, run, 1, body_a);
+                } else {
+                    shade_rows(P, L, len, run, body_b);
+                }
             } else {
-                if constexpr (LANES_B) shade_lanes(P, L, len, run, body_b);
+                if (phase == 0) shade_rows(P, L, len, run, body_a);
                 else shade_rows(P, L, len, run, body_b);
             }
         }
@@ -909,13 +989,13 @@ __device__ __forceinline__ int lists_size(const uint32_t *it)
 {
     const int nw = (int)(uni_u32(it[0]) & 0xffu);
     const int l0 = (int)uni_u32(it[1]), l1 = (int)uni_u32(it[2]), l2 = (int)uni_u32(it[3]), l3 = (int)uni_u32(it[4]);
-    return 8 + ((l0 + 3) & ~3) + ((l1 + 3) & ~3) + ((l2 + 3) & ~3) + ((l3 + 3) & ~3) + nw * 64;
+    return 8 + ((l0 + 3) & ~3) + ((l1 + 3) & ~3) + ((l2 + 3) & ~3) + ((l3 + 3) & ~3) + nw * 72;
 }
 
-// The same iteration driven by a record instead of the tree: body_a over the recorded lists,
-// mid(), body_b over them again.  `at` walks the tile's record stream of `used` words; `lost`
+// The backward's iteration driven by a record instead of the tree: body_a per ray over the
+// recorded lists, once per half of the samples; mid(); body_b over the lists row by row.  `at` walks the tile's record stream of `used` words; `lost`
 // is set when the stream does not hold the items this iteration expects (the caller stops).
-template <bool LANES_A, bool LANES_B, typename BodyA, typename Mid, typename BodyB>
+template <typename BodyA, typename Mid, typename BodyB>
 __device__ __forceinline__ bool slab_replay(const MarchParams &P, const uint32_t *reg, int used, int &at, bool &lost,
                                             const RayState &R, bool need, int &p0, float &found, float &searched_to, BodyA body_a,
                                             Mid mid, BodyB body_b)
@@ -931,7 +1011,11 @@ __device__ __forceinline__ bool slab_replay(const MarchParams &P, const uint32_t
         mid();
         return false;
     }
-    for (int a = start; a < end;) a += replay_lists<true, LANES_A>(P, reg + a, need, p0, body_a);
+    for (int a = start; a < end;) {
+        int dummy = 0;
+        replay_lists<true, 0>(P, reg + a, need, p0, body_a);
+        a += replay_lists<false, 1>(P, reg + a, need, dummy, body_a);
+    }
     const float cover = __uint_as_float(uni_u32(reg[end + 1]));
     found = any_search ? __uint_as_float(reg[end + 4 + threadIdx.x]) : -1.0f;
     searched_to = fminf(R.texit, cover);
@@ -939,7 +1023,7 @@ __device__ __forceinline__ bool slab_replay(const MarchParams &P, const uint32_t
     const bool run = mid();
     if (__any(run)) {
         int dummy = 0;
-        for (int b = start; b < end;) b += replay_lists<false, LANES_B>(P, reg + b, run, dummy, body_b);
+        for (int b = start; b < end;) b += replay_lists<false, -1>(P, reg + b, run, dummy, body_b);
     }
     return run;
 }
@@ -949,7 +1033,8 @@ __device__ __forceinline__ bool slab_replay(const MarchParams &P, const uint32_t
     __shared__ __align__(16) float s_tab[RGX_CCAP * RGX_TAB];         \
     __shared__ uint8_t s_rowlist[4 * RGX_CCAP];                       \
     __shared__ uint32_t s_mask[RGX_CCAP / 32][64];                    \
-    const TileLds L = {s_queue, s_tab, s_rowlist, s_mask}
+    __shared__ uint32_t s_half[2][4][RGX_CCAP / 32];                  \
+    const TileLds L = {s_queue, s_tab, s_rowlist, s_mask, s_half}
 
 // lane -> pixel: row r = lane / 16 is the 4x4 block (r & 1, r >> 1) of the 8x8 tile
 __device__ __forceinline__ void lane_pixel(int px0, int py0, int &px, int &py)
@@ -994,7 +1079,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
 #pragma unroll
             for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
             f3 rdt = dir * fmaf(dt, 0.5f, R.tbuffer); // samples 0..15
-            auto accumulate = [&](const auto &e, bool hit, bool) {
+            auto accumulate = [&](const auto &e, bool hit, bool, auto) {
                 if (hit) {
                     const float4 col = e.prim->rgba4;
                     f3 U, V, W, inv;
@@ -1004,7 +1089,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
                     const float rho = col.w;
 #pragma unroll
                     for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
-                        const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
+                        const float gw = hs.power < hs.cut ? gauss_weight(hs.power) : 0.0f;
                         sg[i] = fmaf(rho, gw, sg[i]);
                         cr[i] = fmaf(col.x, gw, cr[i]);
                         cg[i] = fmaf(col.y, gw, cg[i]);
@@ -1036,7 +1121,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
                 rdt = dir * fmaf(dt, 16.5f, R.tbuffer);
                 return has && R.T > P.m.t_eps;
             };
-            const bool run2 = slab_tables<true, true>(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, accumulate,
+            const bool run2 = slab_tables<WALK_FORWARD>(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, accumulate,
                                           second_half, accumulate);
             if (run2) blend();
             if (need && p0 > 0) {
@@ -1130,7 +1215,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
             for (int i = 0; i < RGX_BUFFER_SIZE; ++i) PA[i] = PB[i] = 0.f;
             const f3 rdt0 = dir * fmaf(dt, 0.5f, tbuffer);
             const f3 rdt1 = dir * fmaf(dt, 16.5f, tbuffer);
-            auto densities = [&](const auto &e, bool hit, bool) {
+            auto densities = [&](const auto &e, bool hit, bool, auto half) {
                 if (hit) {
                     const float4 col = e.prim->rgba4, pos4 = e.prim->pos4;
                     const float rho = col.w;
@@ -1138,19 +1223,11 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
                     f3 U, V, W, inv;
                     float k;
                     e.frame(U, V, W, inv, k);
-                    HitSetup hs = hit_setup(U, V, W, inv, k, pos4, dir, rdt0, dt);
+                    constexpr int base = decltype(half)::value * RGX_CHUNK_SIZE;
+                    HitSetup hs = hit_setup(U, V, W, inv, k, pos4, dir, base ? rdt1 : rdt0, dt);
 #pragma unroll
-                    for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
-                        const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
-                        PA[i] = fmaf(rho, gw, PA[i]);
-                        PB[i] = fmaf(ddc, gw, PB[i]);
-                        hs.power += hs.inc;
-                        hs.inc += hs.inc_st;
-                    }
-                    hs = hit_setup(U, V, W, inv, k, pos4, dir, rdt1, dt);
-#pragma unroll
-                    for (int i = RGX_CHUNK_SIZE; i < RGX_BUFFER_SIZE; ++i) {
-                        const float gw = hs.power < hs.cut ? __expf(-0.5f * hs.power) : 0.0f;
+                    for (int i = base; i < base + RGX_CHUNK_SIZE; ++i) {
+                        const float gw = hs.power < hs.cut ? gauss_weight(hs.power) : 0.0f;
                         PA[i] = fmaf(rho, gw, PA[i]);
                         PB[i] = fmaf(ddc, gw, PB[i]);
                         hs.power += hs.inc;
@@ -1185,7 +1262,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
             };
             // (3) per table entry: moments per lane, row sum, one set of atomics per row
             const f3 xdir_c = dir * fmaf(dt, 16.0f, tbuffer); // slab centre: t_c = tbuffer + 16 dt
-            auto gradients = [&](const auto &e, bool hit, bool live) {
+            auto gradients = [&](const auto &e, bool hit, bool live, auto) {
                 float out[14];
 #pragma unroll
                 for (int c = 0; c < 14; ++c) out[c] = 0.f;
@@ -1216,7 +1293,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
 #pragma unroll
                     for (int i = 0; i < RGX_BUFFER_SIZE; ++i) {
                         const bool on = power < cut && (i < RGX_CHUNK_SIZE || use_second);
-                        const float wd = on ? __expf(-0.5f * power) : 0.0f;
+                        const float wd = on ? gauss_weight(power) : 0.0f;
                         const float y = fmaf(PA[i], dcg, PB[i]) * wd;
                         const float u = (float)i - 15.5f;
                         s0 += y;
@@ -1282,7 +1359,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
         bool lost = false;
         while (__any(R.active) && !lost) {
             iteration([&](bool need, float, float, int &p0, bool &, float &found, float &searched_to, auto a, auto mid, auto b) {
-                return slab_replay<true, false>(P, reg, used, at, lost, R, need, p0, found, searched_to, a, mid, b);
+                return slab_replay(P, reg, used, at, lost, R, need, p0, found, searched_to, a, mid, b);
             });
         }
         if ((lost || at != used) && lane == 0) cn.replay_lost = 1;
@@ -1294,7 +1371,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
         NoRecorder rec;
         while (__any(R.active)) {
             iteration([&](bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to, auto a, auto mid,
-                          auto b) { return slab_tables<true, false>(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, a, mid, b); });
+                          auto b) { return slab_tables<WALK_BACKWARD>(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, a, mid, b); });
         }
     }
     flush_stats(P.stats, cn);
@@ -1334,11 +1411,11 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
         float found = -1.0f, searched_to = 0.f;
         MarchParams Pc = P;
         Pc.m.max_prim_slice = cap;
-        auto record = [&](const auto &e, bool hit, bool) {
+        auto record = [&](const auto &e, bool hit, bool, auto) {
             if (hit) ids[ray * cap + written++] = (int32_t)P.order[e.pid];
         };
         NoRecorder rec;
-        slab_tables<false, false>(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, record, [] { return false; }, record);
+        slab_tables<WALK_ROWS>(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, record, [] { return false; }, record);
     }
     if (valid) counts[ray] = ov ? -p0 : p0;
 }
@@ -1469,8 +1546,8 @@ static int attach_records(MarchParams &P, void *records, size_t records_bytes)
 
 static inline dim3 march_grid(const MarchParams &P)
 {
-    const int ntiles = P.tiles_x * P.tiles_y;
-    return dim3((unsigned)((ntiles + 7) / 8 * 8));
+    const TileGrid g = tile_grid(P.tiles_x, P.tiles_y);
+    return dim3((unsigned)(8 * g.per_xcd * g.bw * RGX_BLOCK_H));
 }
 
 extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,

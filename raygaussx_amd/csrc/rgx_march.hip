@@ -551,6 +551,7 @@ struct Entry {
     const float4 *tab; // LDS table entry (FROM_TABLE only)
     const Prim *prim;
     int32_t pid;       // index in Morton order
+    int slot;          // its slot in the candidate table of the current window
     __device__ __forceinline__ void frame(f3 &U, f3 &V, f3 &W, f3 &inv, float &k) const
     {
         if constexpr (FROM_TABLE) {
@@ -695,7 +696,7 @@ __device__ __forceinline__ void shade_rows(const MarchParams &P, const TileLds &
             const int c = live ? L.rowlist[row * RGX_CCAP + i] : 0;
             const float4 *tab = (const float4 *)(L.tab + c * RGX_TAB);
             const int32_t pid = __float_as_int(L.tab[c * RGX_TAB + 19]);
-            body(Entry<true>{tab, P.prims + pid, pid}, hit, live, Half<0>{});
+            body(Entry<true>{tab, P.prims + pid, pid, c}, hit, live, Half<0>{});
         }
     }
 }
@@ -731,20 +732,25 @@ __device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds 
         }
         const float4 *tab = (const float4 *)(L.tab + c * RGX_TAB);
         const int32_t pid = __float_as_int(L.tab[c * RGX_TAB + 19]);
-        body(Entry<true>{tab, P.prims + pid, pid}, has, has, Half<TAG>{});
+        body(Entry<true>{tab, P.prims + pid, pid, c}, has, has, Half<TAG>{});
     }
 }
 
 // ---------------------------------------------------------------------------
-// Hit-list records.  What the filter produces for a slab iteration -- per 4x4 row the Gaussians
-// some ray of the row hits, per ray its hit bits over that list, per searching ray the first-hit
-// t -- is a few hundred bytes.  The forward can stream it to memory so that the backward replays
-// the same lists instead of sweeping the tree and evaluating the predicate again.  Per tile a region of rec_tile_words 32-bit words:
+// Hit-list records.  What the sweep and the filter produce -- per window the Gaussians of the
+// candidate table, per slab iteration and 4x4 row the table slots some ray of the row hits, per ray
+// its hit bits over that list, per searching ray the first-hit t -- is a few hundred bytes per
+// iteration.  The forward can stream it to memory so that the backward replays the same lists
+// instead of sweeping the tree and evaluating the predicate again.  Per tile a region of
+// rec_tile_words 32-bit words:
 //   word 0: 0 = complete, 1 = the region overflowed (record unusable);  word 1: words used;
-//   from word 4, per iteration:  one LISTS item per table batch, then a TRAIL item
-//   LISTS: {tag | last << 8 | nw, len[4], -, -, -}, pid[pad4(len[r])] for r = 0..3, mask[nw][64],
-//          half[2][4][nw]   (the TileLds arrays of the same names; words past a row's length are junk)
-//   TRAIL: {tag | any_search, cover (float), -, -}, found[64] when any_search
+//   from word 4, per iteration: WINDOW when a table was built, one LISTS per table, then TRAIL
+//   WINDOW: {tag | C, -, -, -}, pid[pad4(C)]            the table's Gaussians, by slot
+//   LISTS:  {tag | last << 8 | nw, len[4], -, -, -}, slot bytes of row r in pad4(len[r]) / 4 words
+//           for r = 0..3, mask[nw][64], half[2][4][nw]   (the TileLds arrays of the same names;
+//           bytes and words past a row's length are junk)
+//   TRAIL:  {tag | any_search, cover (float), -, -}, found[64] when any_search
+#define RGX_REC_WINDOW 0x57000000u
 #define RGX_REC_LISTS 0x4C000000u
 #define RGX_REC_TRAIL 0x54000000u
 
@@ -754,6 +760,21 @@ struct Recorder {
     int cap;        // words in the region
     bool ovf;       // the region is exhausted
     __device__ __forceinline__ bool on() const { return reg != nullptr && !ovf; }
+    // room for an item and the iteration's trailer?
+    __device__ __forceinline__ bool fits(int size)
+    {
+        if (off + size + 72 > cap) ovf = true;
+        return !ovf;
+    }
+
+    __device__ __forceinline__ void write_window(const TileLds &L, int C)
+    {
+        if (!on() || !fits(4 + ((C + 3) & ~3))) return;
+        uint32_t *it = reg + off;
+        if (threadIdx.x == 0) it[0] = RGX_REC_WINDOW | (uint32_t)C;
+        for (int i = threadIdx.x; i < C; i += 64) it[4 + i] = __float_as_uint(L.tab[i * RGX_TAB + 19]);
+        off += 4 + ((C + 3) & ~3);
+    }
 
     __device__ __forceinline__ void write_lists(const TileLds &L, int len, bool last)
     {
@@ -762,21 +783,18 @@ struct Recorder {
         const int l0 = __builtin_amdgcn_readlane(len, 0), l1 = __builtin_amdgcn_readlane(len, 16);
         const int l2 = __builtin_amdgcn_readlane(len, 32), l3 = __builtin_amdgcn_readlane(len, 48);
         const int nw = (max(max(l0, l1), max(l2, l3)) + 31) >> 5;
-        const int p0 = (l0 + 3) & ~3, p1 = (l1 + 3) & ~3, p2 = (l2 + 3) & ~3, p3 = (l3 + 3) & ~3;
-        const int size = 8 + p0 + p1 + p2 + p3 + nw * 72;
-        if (off + size + 72 > cap) { // always leave room for the iteration's trailer
-            ovf = true;
-            return;
-        }
+        const int q0 = (l0 + 3) >> 2, q1 = (l1 + 3) >> 2, q2 = (l2 + 3) >> 2, q3 = (l3 + 3) >> 2;
+        const int size = 8 + q0 + q1 + q2 + q3 + nw * 72;
+        if (!fits(size)) return;
         uint32_t *it = reg + off;
         if (lane == 0) {
             it[0] = RGX_REC_LISTS | (last ? 0x100u : 0u) | (uint32_t)nw;
             it[1] = (uint32_t)l0; it[2] = (uint32_t)l1; it[3] = (uint32_t)l2; it[4] = (uint32_t)l3;
         }
-        const int base = 8 + (row > 0 ? p0 : 0) + (row > 1 ? p1 : 0) + (row > 2 ? p2 : 0);
-        for (int i = lane & 15; i < len; i += 16)
-            it[base + i] = __float_as_uint(L.tab[L.rowlist[row * RGX_CCAP + i] * RGX_TAB + 19]);
-        const int mbase = 8 + p0 + p1 + p2 + p3;
+        const int base = 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0);
+        const uint32_t *slots = (const uint32_t *)(L.rowlist + row * RGX_CCAP);
+        for (int i = lane & 15; i < ((len + 3) >> 2); i += 16) it[base + i] = slots[i];
+        const int mbase = 8 + q0 + q1 + q2 + q3;
         for (int w = 0; w < nw; ++w) it[mbase + w * 64 + lane] = L.mask[w][lane];
         if ((lane & 15) < 2) // two lanes per row: one per half
             for (int w = 0; w < nw; ++w) it[mbase + nw * 64 + ((lane & 15) * 4 + row) * nw + w] = L.half[lane & 15][row][w];
@@ -806,6 +824,7 @@ struct Recorder {
 
 // Stand-in where nothing is recorded.
 struct NoRecorder {
+    __device__ __forceinline__ void write_window(const TileLds &, int) {}
     __device__ __forceinline__ void write_lists(const TileLds &, int, bool) {}
     __device__ __forceinline__ void write_trailer(bool, float, float) {}
     __device__ __forceinline__ void finish() {}
@@ -813,39 +832,77 @@ struct NoRecorder {
 
 __device__ __forceinline__ uint32_t uni_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
-// Replays one LISTS item as shade_rows (the four rows walk their recorded lists in lock step) or,
-// with HALF >= 0, as shade_lanes<HALF> (every ray walks its own hits) does on a live table.  COUNT
-// adds the lane's hits to p0.  Returns the item's size.
-template <bool COUNT, int HALF, typename Body>
-__device__ __forceinline__ int replay_lists(const MarchParams &P, const uint32_t *it, bool run, int &p0, Body body)
+// The replaying backward keeps, per tile, the gradient sums of the current window's Gaussians in
+// LDS (one column of 14 per table slot): a row's share is added there with LDS atomics, and the
+// sums go to memory once per window instead of once per row, slab and Gaussian.
+struct ReplayLds {
+    float *acc;        // [14][RGX_CCAP], component-major so that different slots fall in different banks
+    uint32_t *pid;     // [RGX_CCAP]: the window's Gaussians by slot
+    uint32_t *touched; // [RGX_CCAP / 32]: slots with something in acc
+};
+
+__device__ __forceinline__ void replay_flush(const MarchParams &P, const ReplayLds &RL)
+{
+    __syncthreads();
+    for (int slot = threadIdx.x; slot < RGX_CCAP; slot += 64) {
+        if ((RL.touched[slot >> 5] >> (slot & 31)) & 1u) {
+            float *dst = P.gbuf + (int64_t)RL.pid[slot] * 16;
+#pragma unroll
+            for (int c = 0; c < 14; ++c) {
+                unsafeAtomicAdd(dst + c, RL.acc[c * RGX_CCAP + slot]);
+                RL.acc[c * RGX_CCAP + slot] = 0.f;
+            }
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < RGX_CCAP / 32) RL.touched[threadIdx.x] = 0u;
+    __syncthreads();
+}
+
+// Makes the WINDOW item at `at` the current window (sums of the previous one go to memory first).
+__device__ __forceinline__ void replay_window(const MarchParams &P, const ReplayLds &RL, const uint32_t *reg, int at, int &win_at)
+{
+    if (at == win_at) return;
+    replay_flush(P, RL);
+    const int C = (int)(uni_u32(reg[at]) & 0xffffu);
+    for (int i = threadIdx.x; i < C && i < RGX_CCAP; i += 64) RL.pid[i] = reg[at + 4 + i];
+    win_at = at;
+    __syncthreads();
+}
+
+// Replays one LISTS item.  WALK_ROWS: as shade_rows (the four rows walk their recorded lists in lock
+// step); WALK 0 / 1: as shade_lanes over one half's entries; WALK_LANES_ALL: every ray walks all
+// its hits.  COUNT adds the lane's hits to p0.  Returns the item's size.
+enum { WALK_LANES_ALL = 2, WALK_ROWS_ALL = 3 };
+template <bool COUNT, int WALK, typename Body>
+__device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLds &RL, const uint32_t *it, bool run, int &p0, Body body)
 {
     const int lane = threadIdx.x, row = lane >> 4;
     const int nw = (int)(uni_u32(it[0]) & 0xffu);
     const int l0 = (int)uni_u32(it[1]), l1 = (int)uni_u32(it[2]), l2 = (int)uni_u32(it[3]), l3 = (int)uni_u32(it[4]);
-    const int q0 = (l0 + 3) & ~3, q1 = (l1 + 3) & ~3, q2 = (l2 + 3) & ~3, q3 = (l3 + 3) & ~3;
+    const int q0 = (l0 + 3) >> 2, q1 = (l1 + 3) >> 2, q2 = (l2 + 3) >> 2, q3 = (l3 + 3) >> 2;
     const int len = row == 0 ? l0 : row == 1 ? l1 : row == 2 ? l2 : l3;
-    const uint32_t *pids = it + 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0);
+    const uint8_t *slots = (const uint8_t *)(it + 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0));
     const uint32_t *masks = it + 8 + q0 + q1 + q2 + q3 + lane; // word w of this lane: masks[w * 64]
-    if constexpr (HALF >= 0) {
+    if constexpr (WALK != WALK_ROWS_ALL) {
         const int nwr = run ? (len + 31) >> 5 : 0; // words of this lane's row; later words are not its own
-        const uint32_t *half = it + 8 + q0 + q1 + q2 + q3 + nw * 64 + (HALF * 4 + row) * nw;
+        const uint32_t *half = it + 8 + q0 + q1 + q2 + q3 + nw * 64 + ((WALK & 1) * 4 + row) * nw;
+        auto word = [&](int w) { return WALK == WALK_LANES_ALL ? masks[w * 64] : masks[w * 64] & half[w]; };
         if (COUNT)
             for (int w = 0; w < nwr; ++w) p0 += __popc(masks[w * 64]);
         int w = 0;
-        uint32_t bits = nwr > 0 ? masks[0] & half[0] : 0u;
+        uint32_t bits = nwr > 0 ? word(0) : 0u;
         for (;;) {
-            while (bits == 0u && w + 1 < nwr) {
-                ++w;
-                bits = masks[w * 64] & half[w];
-            }
+            while (bits == 0u && w + 1 < nwr) bits = word(++w);
             const bool has = bits != 0u;
             if (!__any(has)) break;
-            int32_t pid = 0;
+            int slot = 0;
             if (has) {
-                pid = (int32_t)pids[w * 32 + __builtin_ctz(bits)];
+                slot = slots[w * 32 + __builtin_ctz(bits)];
                 bits &= bits - 1u;
             }
-            body(Entry<false>{nullptr, P.prims + pid, pid}, has, has, Half<(HALF < 0 ? 0 : HALF)>{});
+            const int32_t pid = (int32_t)RL.pid[slot];
+            body(Entry<false>{nullptr, P.prims + pid, pid, slot}, has, has, Half<(WALK & 1)>{});
         }
     } else {
         const int maxlen = max(max(l0, l1), max(l2, l3));
@@ -856,8 +913,9 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const uint32_t
             const bool hit = run && live && ((bits >> (i & 31)) & 1u);
             if (COUNT && hit) ++p0;
             if (__ballot(hit)) {
-                const int32_t pid = live ? (int32_t)pids[i] : 0;
-                body(Entry<false>{nullptr, P.prims + pid, pid}, hit, live, Half<0>{});
+                const int slot = live ? slots[i] : 0;
+                const int32_t pid = (int32_t)RL.pid[slot];
+                body(Entry<false>{nullptr, P.prims + pid, pid, slot}, hit, live, Half<0>{});
             }
         }
     }
@@ -940,6 +998,7 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                 first = false;
                 more = !done;
             }
+            if (phase == 0 && !reuse) rec.write_window(L, C);
             if (phase == 0 || !Wn.resident) {
                 // phase 0 asks the lane's real question; a phase-1 re-filter only recounts the slab hits
                 const float cover = Wn.resident ? Wn.hi : t1; // this iteration's tables cover [t0, cover]
@@ -989,44 +1048,73 @@ __device__ __forceinline__ int lists_size(const uint32_t *it)
 {
     const int nw = (int)(uni_u32(it[0]) & 0xffu);
     const int l0 = (int)uni_u32(it[1]), l1 = (int)uni_u32(it[2]), l2 = (int)uni_u32(it[3]), l3 = (int)uni_u32(it[4]);
-    return 8 + ((l0 + 3) & ~3) + ((l1 + 3) & ~3) + ((l2 + 3) & ~3) + ((l3 + 3) & ~3) + nw * 72;
+    return 8 + ((l0 + 3) >> 2) + ((l1 + 3) >> 2) + ((l2 + 3) >> 2) + ((l3 + 3) >> 2) + nw * 72;
 }
 
-// The backward's iteration driven by a record instead of the tree: body_a per ray over the
-// recorded lists, once per half of the samples; mid(); body_b over the lists row by row.  `at` walks the tile's record stream of `used` words; `lost`
-// is set when the stream does not hold the items this iteration expects (the caller stops).
-template <typename BodyA, typename Mid, typename BodyB>
-__device__ __forceinline__ bool slab_replay(const MarchParams &P, const uint32_t *reg, int used, int &at, bool &lost,
-                                            const RayState &R, bool need, int &p0, float &found, float &searched_to, BodyA body_a,
-                                            Mid mid, BodyB body_b)
-{
-    const int start = at;
-    int end = at; // one past the iteration's last LISTS item
-    while (end + 8 <= used && (uni_u32(reg[end]) & 0xff000000u) == RGX_REC_LISTS && end + lists_size(reg + end) <= used)
-        end += lists_size(reg + end);
-    const uint32_t tr = end + 4 <= used ? uni_u32(reg[end]) : 0u;
-    const bool any_search = tr & 1u;
-    if ((tr & 0xff000000u) != RGX_REC_TRAIL || end + 4 + (any_search ? 64 : 0) > used) {
-        lost = true;
-        mid();
-        return false;
-    }
-    for (int a = start; a < end;) {
+// Walks the record stream of one tile for the backward.
+struct Replayer {
+    const uint32_t *reg; // the tile's region
+    int used;            // words the forward wrote
+    int at;              // next item
+    int win_at;          // the WINDOW item whose Gaussians sit in RL.pid (-1: none yet)
+    bool lost;           // the stream did not hold the items an iteration expects (the caller stops)
+    ReplayLds RL;
+
+    // The backward's iteration driven by the record instead of the tree: body_a per ray over the
+    // recorded lists, once per half of the samples; mid(); body_b over the lists row by row.
+    template <typename BodyA, typename Mid, typename BodyB>
+    __device__ __forceinline__ bool slab(const MarchParams &P, const RayState &R, bool need, int &p0, float &found,
+                                         float &searched_to, BodyA body_a, Mid mid, BodyB body_b)
+    {
+        const int start = at;
+        int end = at; // the iteration's TRAIL item
+        for (;;) {
+            if (end + 4 > used) break;
+            const uint32_t head = uni_u32(reg[end]);
+            int size;
+            if ((head & 0xff000000u) == RGX_REC_WINDOW) size = 4 + (((int)(head & 0xffffu) + 3) & ~3);
+            else if ((head & 0xff000000u) == RGX_REC_LISTS && end + 8 <= used) size = lists_size(reg + end);
+            else break;
+            if (end + size > used) break;
+            end += size;
+        }
+        const uint32_t tr = end + 4 <= used ? uni_u32(reg[end]) : 0u;
+        const bool any_search = tr & 1u;
+        if ((tr & 0xff000000u) != RGX_REC_TRAIL || end + 4 + (any_search ? 64 : 0) > used) {
+            lost = true;
+            mid();
+            return false;
+        }
         int dummy = 0;
-        replay_lists<true, 0>(P, reg + a, need, p0, body_a);
-        a += replay_lists<false, 1>(P, reg + a, need, dummy, body_a);
+        for (int a = start; a < end;) {
+            const uint32_t head = uni_u32(reg[a]);
+            if ((head & 0xff000000u) == RGX_REC_WINDOW) {
+                replay_window(P, RL, reg, a, win_at);
+                a += 4 + (((int)(head & 0xffffu) + 3) & ~3);
+            } else {
+                replay_lists<true, 0>(P, RL, reg + a, need, p0, body_a);
+                a += replay_lists<false, 1>(P, RL, reg + a, need, dummy, body_a);
+            }
+        }
+        const float cover = __uint_as_float(uni_u32(reg[end + 1]));
+        found = any_search ? __uint_as_float(reg[end + 4 + threadIdx.x]) : -1.0f;
+        searched_to = fminf(R.texit, cover);
+        at = end + 4 + (any_search ? 64 : 0);
+        const bool run = mid();
+        if (__any(run)) {
+            for (int b = start; b < end;) {
+                const uint32_t head = uni_u32(reg[b]);
+                if ((head & 0xff000000u) == RGX_REC_WINDOW) {
+                    replay_window(P, RL, reg, b, win_at);
+                    b += 4 + (((int)(head & 0xffffu) + 3) & ~3);
+                } else {
+                    b += replay_lists<false, WALK_ROWS_ALL>(P, RL, reg + b, run, dummy, body_b);
+                }
+            }
+        }
+        return run;
     }
-    const float cover = __uint_as_float(uni_u32(reg[end + 1]));
-    found = any_search ? __uint_as_float(reg[end + 4 + threadIdx.x]) : -1.0f;
-    searched_to = fminf(R.texit, cover);
-    at = end + 4 + (any_search ? 64 : 0);
-    const bool run = mid();
-    if (__any(run)) {
-        int dummy = 0;
-        for (int b = start; b < end;) b += replay_lists<false, -1>(P, reg + b, run, dummy, body_b);
-    }
-    return run;
-}
+};
 
 #define RGX_TILE_LDS()                                                \
     __shared__ int32_t s_queue[RGX_QCAP];                             \
@@ -1183,6 +1271,14 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
         if (uni_u32(reg[0]) == 0u) return; // replayed
     }
     const int lane = threadIdx.x;
+    __shared__ float s_acc[REPLAY ? 14 * RGX_CCAP : 1];
+    __shared__ uint32_t s_pid[REPLAY ? RGX_CCAP : 1], s_touched[REPLAY ? RGX_CCAP / 32 : 1];
+    const ReplayLds RL = {s_acc, s_pid, s_touched};
+    if constexpr (REPLAY) {
+        for (int i = lane; i < 14 * RGX_CCAP; i += 64) s_acc[i] = 0.f;
+        if (lane < RGX_CCAP / 32) s_touched[lane] = 0u;
+        __syncthreads();
+    }
     int px, py;
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
@@ -1332,13 +1428,26 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
                     out[13] = -4 * qw * d1.x + 2 * qx * d1.y + 2 * qy * d1.z - 2 * qx * d2.x - 4 * qw * d2.y + 2 * qz * d2.z +
                               2 * qy * d3.x + 2 * qz * d3.y;
                 }
-                const uint64_t bal = __ballot(hit);
+                if constexpr (REPLAY) {
+                    // summed over the row's rays, one lane per row adds to the window's sums in LDS
+                    const uint64_t bal = __ballot(hit);
 #pragma unroll
-                for (int c = 0; c < 14; ++c) out[c] = row_sum(out[c]);
-                if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
-                    float *dst = P.gbuf + (int64_t)pid * 16;
+                    for (int c = 0; c < 14; ++c) out[c] = row_sum(out[c]);
+                    if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
+                        atomicOr(&s_touched[e.slot >> 5], 1u << (e.slot & 31));
 #pragma unroll
-                    for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, out[c]);
+                        for (int c = 0; c < 14; ++c) unsafeAtomicAdd(&s_acc[c * RGX_CCAP + e.slot], out[c]);
+                    }
+                } else {
+                    // summed over the row's rays, one lane per row adds to memory
+                    const uint64_t bal = __ballot(hit);
+#pragma unroll
+                    for (int c = 0; c < 14; ++c) out[c] = row_sum(out[c]);
+                    if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
+                        float *dst = P.gbuf + (int64_t)pid * 16;
+#pragma unroll
+                        for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, out[c]);
+                    }
                 }
             };
             const bool has = drive(need, tlo, thi, p0, ov, found, searched_to, densities, prefix, gradients);
@@ -1354,15 +1463,14 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
     };
 
     if constexpr (REPLAY) {
-        const int used = min((int)uni_u32(reg[1]), P.rec_tile_words);
-        int at = 4;
-        bool lost = false;
-        while (__any(R.active) && !lost) {
+        Replayer rp = {reg, min((int)uni_u32(reg[1]), P.rec_tile_words), 4, -1, false, RL};
+        while (__any(R.active) && !rp.lost) {
             iteration([&](bool need, float, float, int &p0, bool &, float &found, float &searched_to, auto a, auto mid, auto b) {
-                return slab_replay(P, reg, used, at, lost, R, need, p0, found, searched_to, a, mid, b);
+                return rp.slab(P, R, need, p0, found, searched_to, a, mid, b);
             });
         }
-        if ((lost || at != used) && lane == 0) cn.replay_lost = 1;
+        replay_flush(P, RL);
+        if ((rp.lost || rp.at != rp.used) && lane == 0) cn.replay_lost = 1;
     } else {
         RGX_TILE_LDS();
         Frustum F;

@@ -600,6 +600,8 @@ struct LaneQuery {
     float slo, shi;
     int cap;        // max_prim_slice
     float tmid;     // tbuffer + 16 dt: where the slab's second 16 samples begin
+    int part;       // 0: all hits of [tlo, thi]; 1: only those reaching the first 16 samples; 2: only those
+                    // reaching the second 16, of which the ones that also reach the first are not counted again
 };
 
 // Filter: every lane tests the table entries whose distance shell meets [t0, t1] (the union of
@@ -646,12 +648,14 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
                     if (Q.search) {
                         if (segment_hit(r1, r2, Q.slo, Q.shi, t)) found = found < 0.0f ? t : fminf(found, t);
                     } else if (segment_hit(r1, r2, Q.tlo, Q.thi, t)) {
-                        if (p0 >= Q.cap) ov = true;
-                        else {
-                            ++p0;
+                        const bool f = r1 < Q.tmid, g = r2 > Q.tmid;
+                        const bool counts = Q.part != 2 || !f;
+                        if (counts && p0 >= Q.cap) ov = true;
+                        else if (Q.part == 0 || (Q.part == 1 ? f : g)) {
+                            p0 += counts;
                             hit = true;
-                            in_first = r1 < Q.tmid ? 1u : 0u;
-                            in_second = r2 > Q.tmid ? 1u : 0u;
+                            in_first = f ? 1u : 0u;
+                            in_second = g ? 1u : 0u;
                         }
                     }
                 }
@@ -928,7 +932,8 @@ struct Window {
     float hi;
     int n;
     bool resident;
-    int k; // slabs to look ahead when a window is built
+    int k;        // slabs to look ahead when a window is built
+    bool crowded; // the last iteration's Gaussians did not fit one table
 };
 
 __device__ __forceinline__ void frustum_range(Frustum &F, float t0, float t1)
@@ -943,7 +948,7 @@ __device__ __forceinline__ void frustum_range(Frustum &F, float t0, float t1)
 //   phase 0  make the table cover the wave's intervals (reuse the resident window, or sweep a new
 //            one looking Wn.k slabs ahead, or -- when even this iteration's own range overflows
 //            the table -- walk it in table-sized batches), filter, body_a over the row lists;
-//   mid()    per lane, between the phases; returns whether the lane takes part in phase 1;
+//   mid(split) per lane, between the phases; returns whether the lane takes part in phase 1;
 //   phase 1  body_b over the same row lists, or over freshly swept and filtered batches when the
 //            candidates did not fit one table.
 // WALK_FORWARD: body_a per ray over the entries reaching the first 16 samples, body_b per ray over
@@ -959,15 +964,28 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
     const bool srch = R.active && R.searching, want = need || srch;
     const float t0 = wave_min_all(want ? tlo : INFINITY), t1 = wave_max_all(want ? thi : -INFINITY);
     const bool any_search = __any(srch);
-    int len = 0, q0 = 0;
+    const float tmid = fmaf(R.dt, (float)RGX_CHUNK_SIZE, R.tbuffer);
+    // Where slabs hold more Gaussians than a table (the previous iteration found so), a forward
+    // that records nothing sweeps each half of the slab's depth range for its own phase instead
+    // of the whole range twice: phase 0 takes the Gaussians that reach the first 16 samples,
+    // phase 1 those that reach the second 16, and a Gaussian of both halves is counted once.
+    const bool split = WALK == WALK_FORWARD && std::is_same<Rec, NoRecorder>::value && Wn.crowded && __any(need);
+    int len = 0, q0 = 0, seen = 0;
     bool run = need, qov = false;
     for (int phase = 0; phase < 2; ++phase) {
-        const bool reuse = Wn.resident && t1 <= Wn.hi;
+        const bool reuse = !split && Wn.resident && t1 <= Wn.hi;
+        float lo = t0, hi = t1; // depth range of this phase's tables
+        if (split) {
+            if (phase == 0) hi = wave_max_all(need ? fminf(thi, tmid) : -INFINITY); // searching rays look as far as that
+            else lo = wave_min_all(run && tmid < thi ? fmaxf(tlo, tmid) : INFINITY), hi = wave_max_all(run ? thi : -INFINITY);
+            if (!(lo <= hi)) break; // no ray reaches into the second half
+        }
         Sweep S = {0};
         if (!reuse) {
-            float wend = t1;
-            if (phase == 0 && Wn.k > 1) wend = fmaxf(t1, wave_max_all(want ? tlo + (float)Wn.k * R.slab_spacing : -INFINITY));
-            frustum_range(F, t0, wend);
+            float wend = hi;
+            if (!split && phase == 0 && Wn.k > 1)
+                wend = fmaxf(t1, wave_max_all(want ? tlo + (float)Wn.k * R.slab_spacing : -INFINITY));
+            frustum_range(F, lo, wend);
             sweep_begin(P, S, L.queue);
         }
         bool first = true, more = true;
@@ -979,11 +997,14 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
             } else {
                 bool done;
                 C = sweep_next(P, S, F, L.queue, L.tab, done, cn);
-                if (phase == 0 && first) {
+                if (split) {
+                    seen += C;
+                } else if (phase == 0 && first) {
                     if (done) {
                         Wn.hi = F.t1;
                         Wn.n = C;
                         Wn.resident = true;
+                        Wn.crowded = false;
                         if (C > (RGX_CCAP * 3) / 4) Wn.k = Wn.k > 1 ? Wn.k / 2 : 1;
                         else if (C < RGX_CCAP / 3 && Wn.k < 32) Wn.k *= 2;
                     } else if (Wn.k > 1) {
@@ -993,30 +1014,34 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                         continue;
                     } else {
                         Wn.resident = false;
+                        Wn.crowded = true;
                     }
                 }
                 first = false;
                 more = !done;
             }
             if (phase == 0 && !reuse) rec.write_window(L, C);
-            if (phase == 0 || !Wn.resident) {
+            if (phase == 0 || !Wn.resident || split) {
                 // phase 0 asks the lane's real question; a phase-1 re-filter only recounts the slab hits
-                const float cover = Wn.resident ? Wn.hi : t1; // this iteration's tables cover [t0, cover]
+                const float cover = split ? hi : (Wn.resident ? Wn.hi : t1); // this iteration's tables cover [t0, cover]
                 const LaneQuery Q = {R.dir, run, tlo, thi, phase == 0 && srch, R.tbuffer, fminf(R.texit, cover), P.m.max_prim_slice,
-                                     fmaf(R.dt, (float)RGX_CHUNK_SIZE, R.tbuffer)};
-                int cnt = phase == 0 ? p0 : q0;
-                bool cut = phase == 0 ? ov : qov;
+                                     tmid, split ? phase + 1 : 0};
+                const bool real = phase == 0 || split; // counts into the lane's own p0 / ov
+                int cnt = real ? p0 : q0;
+                bool cut = real ? ov : qov;
                 float best = phase == 0 ? found : -1.0f;
-                filter_table(L, C, t0, (phase == 0 && any_search) ? cover : t1, Q, cnt, cut, best, len, cn);
-                if (phase == 0) {
+                filter_table(L, C, lo, (phase == 0 && any_search) ? cover : hi, Q, cnt, cut, best, len, cn);
+                if (real) {
                     p0 = cnt;
                     ov = cut;
-                    found = best;
-                    searched_to = Q.shi;
-                    rec.write_lists(L, len, !more);
                 } else {
                     q0 = cnt;
                     qov = cut;
+                }
+                if (phase == 0) {
+                    found = best;
+                    searched_to = fmaxf(Q.slo, Q.shi); // a split phase may end before a searching ray's start
+                    rec.write_lists(L, len, !more);
                 }
             }
             if constexpr (WALK == WALK_FORWARD) {
@@ -1035,11 +1060,12 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
             }
         }
         if (phase == 0) {
-            rec.write_trailer(any_search, Wn.resident ? Wn.hi : t1, found);
-            run = mid();
+            rec.write_trailer(any_search, split ? hi : (Wn.resident ? Wn.hi : t1), found);
+            run = mid(split);
             if (!__any(run)) break;
         }
     }
+    if (split && seen < RGX_CCAP / 2) Wn.crowded = false; // sparse again: go back to resident windows
     return run;
 }
 
@@ -1082,7 +1108,7 @@ struct Replayer {
         const bool any_search = tr & 1u;
         if ((tr & 0xff000000u) != RGX_REC_TRAIL || end + 4 + (any_search ? 64 : 0) > used) {
             lost = true;
-            mid();
+            mid(false);
             return false;
         }
         int dummy = 0;
@@ -1100,7 +1126,7 @@ struct Replayer {
         found = any_search ? __uint_as_float(reg[end + 4 + threadIdx.x]) : -1.0f;
         searched_to = fminf(R.texit, cover);
         at = end + 4 + (any_search ? 64 : 0);
-        const bool run = mid();
+        const bool run = mid(false);
         if (__any(run)) {
             for (int b = start; b < end;) {
                 const uint32_t head = uni_u32(reg[b]);
@@ -1153,7 +1179,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
     ray_begin<false>(P, px, py, valid, R);
     const f3 dir = R.dir;
     float Cr = 0.f, Cg = 0.f, Cb = 0.f;
-    Window Wn = {0.f, 0, false, 4};
+    Window Wn = {0.f, 0, false, 4, false};
 
     while (__any(R.active)) {
         float tlo, thi;
@@ -1200,8 +1226,8 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
                     R.T *= w;
                 }
             };
-            auto second_half = [&]() {
-                const bool has = need && p0 > 0;
+            auto second_half = [&](bool split) { // split: the hits of the second half are not known yet
+                const bool has = need && (p0 > 0 || split);
                 if (has) blend();
                 // samples 16..31, only for rays still above the transmittance floor (gaussians_aabb.cu:190)
 #pragma unroll
@@ -1335,7 +1361,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
             // it always covers all 32 samples (330-352)
             float T_after = R.T, D_after = D;
             bool use_second = true; // transmittance at the chunk boundary gates the second chunk (398)
-            auto prefix = [&]() {
+            auto prefix = [&](bool) {
                 const bool has = need && p0 > 0;
                 if (has) {
                     float T_mid = R.T;
@@ -1475,7 +1501,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
         RGX_TILE_LDS();
         Frustum F;
         frustum_planes(P.cam, px0, py0, F);
-        Window Wn = {0.f, 0, false, 4};
+        Window Wn = {0.f, 0, false, 4, false};
         NoRecorder rec;
         while (__any(R.active)) {
             iteration([&](bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to, auto a, auto mid,
@@ -1515,7 +1541,7 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
         R.tbuffer = tlo;
         R.texit = thi;
         R.slab_spacing = 0.f;
-        Window Wn = {0.f, 0, false, 1};
+        Window Wn = {0.f, 0, false, 1, false};
         float found = -1.0f, searched_to = 0.f;
         MarchParams Pc = P;
         Pc.m.max_prim_slice = cap;
@@ -1523,7 +1549,7 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
             if (hit) ids[ray * cap + written++] = (int32_t)P.order[e.pid];
         };
         NoRecorder rec;
-        slab_tables<WALK_ROWS>(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, record, [] { return false; }, record);
+        slab_tables<WALK_ROWS>(Pc, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, record, [](bool) { return false; }, record);
     }
     if (valid) counts[ray] = ov ? -p0 : p0;
 }

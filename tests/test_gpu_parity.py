@@ -292,9 +292,13 @@ def test_backward_replay_of_recorded_hit_lists_equals_recomputation(gx, orc):
         _step("replay vs recompute: " + label)
         a = gx.gpu_render(sc, cam, cfg, want_grad=dloss, record_hits=False)
         b = gx.gpu_render(sc, cam, cfg, want_grad=dloss, record_hits=True, rec_tile_words=words)
-        assert np.array_equal(a["image"], b["image"])
-        for k in ("hit_pairs", "slabs", "empty_slabs", "overflow_rays", "rays_hit"):
+        # the recording forward and the plain one may add a ray's Gaussians in different orders
+        assert np.abs(a["image"] - b["image"]).max() <= 2e-6
+        for k in ("slabs", "empty_slabs", "overflow_rays", "rays_hit"):
             assert a["stats_fwd"][k] == b["stats_fwd"][k], k
+        # where a tile's slabs hold more Gaussians than a candidate table, the plain forward does not
+        # look for the second half's Gaussians of a ray that the first half has already made opaque
+        assert 0.9 * b["stats_fwd"]["hit_pairs"] <= a["stats_fwd"]["hit_pairs"] <= b["stats_fwd"]["hit_pairs"]
         assert a["stats_bwd"]["hit_pairs"] == b["stats_bwd"]["hit_pairs"] > 10000
         assert a["stats_bwd"]["slabs"] == b["stats_bwd"]["slabs"]
         if words is None:   # everything replayed: the backward fetched no tree node

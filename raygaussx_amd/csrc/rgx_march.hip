@@ -1286,7 +1286,7 @@ __device__ __forceinline__ float row_sum(float v)
 // recurrence exactly.  The 14 gradient words of a Gaussian are summed over the 16
 // rays of a row with DPP adds before one lane per row adds them to memory.
 template <bool REPLAY>
-__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchParams P)
+__device__ __forceinline__ void march_bwd(const MarchParams &P)
 {
     int px0, py0, tile;
     if (!tile_origin(P, px0, py0, &tile)) return; // whole wave
@@ -1511,6 +1511,11 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
     flush_stats(P.stats, cn);
 }
 
+// The backward that searches the tree, and the one that replays the forward's record.  (Three
+// waves per SIMD with some spilling measured faster for the replay than two waves without.)
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchParams P) { march_bwd<false>(P); }
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay(const MarchParams P) { march_bwd<true>(P); }
+
 // Test hook for the cooperative collect: per pixel a segment [tlo, thi] (thi < tlo = pixel idle);
 // writes each ray's hit count (negated when cut at cap) and the INPUT indices of its hits.
 __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const float *__restrict__ seg_lo,
@@ -1722,10 +1727,10 @@ extern "C" int rgx_march_backward(const void *ws, const RgxCamera *cam, const Rg
     void *span = rgx_span_begin(RGX_T_MARCH_BWD, s);
     if (P.records) {
         // tiles with a complete record replay it; the few whose record overflowed are recomputed
-        hipLaunchKernelGGL(k_march_bwd<true>, march_grid(P), dim3(64), 0, s, P);
+        hipLaunchKernelGGL(k_march_bwd_replay, march_grid(P), dim3(64), 0, s, P);
         P.only_overflow = 1;
     }
-    hipLaunchKernelGGL(k_march_bwd<false>, march_grid(P), dim3(64), 0, s, P);
+    hipLaunchKernelGGL(k_march_bwd, march_grid(P), dim3(64), 0, s, P);
     rgx_span_end(span, s);
     span = rgx_span_begin(RGX_T_UNPERMUTE, s);
     hipLaunchKernelGGL(k_unpermute_grads, grid_for(n, 256), dim3(256), 0, s, (const float4 *)P.gbuf, P.order, n, ddens, drgb,

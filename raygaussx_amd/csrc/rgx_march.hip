@@ -185,6 +185,8 @@ __device__ int collect(const MarchParams &P, f3 o, f3 dir, float tlo, float thi,
 struct Frustum {
     f3 o;
     f3 n[4]; // unit normals pointing out of the frustum
+    f3 dc;       // the tile's central direction
+    float delta; // no ray of the tile is further than this angle from dc
     float t0, t1, pad;
 };
 
@@ -208,9 +210,16 @@ __device__ __forceinline__ void frustum_planes(const RgxCamera &cam, int px0, in
     F.n[1] = plane_normal(d10, d11, in);
     F.n[2] = plane_normal(d00, d10, in);
     F.n[3] = plane_normal(d01, d11, in);
+    F.dc = in * (1.0f / sqrtf(dot3(in, in)));
+    // the rays' directions lie, before normalisation, in a plane quadrilateral with these four as
+    // corners, so the largest angle to dc is at a corner; |d - dc| = 2 sin(angle / 2)
+    const f3 e00 = d00 - F.dc, e10 = d10 - F.dc, e01 = d01 - F.dc, e11 = d11 - F.dc;
+    F.delta = 1.02f * sqrtf(fmaxf(fmaxf(dot3(e00, e00), dot3(e10, e10)), fmaxf(dot3(e01, e01), dot3(e11, e11)))) + 1e-6f;
     // the planes are the same in every lane: keep them in scalar registers
     auto uni = [](float v) { return __int_as_float(__builtin_amdgcn_readfirstlane(__float_as_int(v))); };
     F.o = mk3(uni(F.o.x), uni(F.o.y), uni(F.o.z));
+    F.dc = mk3(uni(F.dc.x), uni(F.dc.y), uni(F.dc.z));
+    F.delta = uni(F.delta);
 #pragma unroll
     for (int k = 0; k < 4; ++k) F.n[k] = mk3(uni(F.n[k].x), uni(F.n[k].y), uni(F.n[k].z));
 }
@@ -304,9 +313,20 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
             // semi-axes of the k-sigma ellipsoid: k * scale = 1 / inv_inter
             const f3 ax = mk3(1.0f / p.inv_inter4.x, 1.0f / p.inv_inter4.y, 1.0f / p.inv_inter4.z);
             const float dist = sqrtf(dot3(O, O));
-            const float rad = fmaxf(ax.x, fmaxf(ax.y, ax.z)) * 1.001f + 1e-5f * dist + F.pad;
-            dmin = dist - rad;
-            dmax = dist + rad;
+            const float amax = fmaxf(ax.x, fmaxf(ax.y, ax.z));
+            const float rad = amax * 1.001f + 1e-5f * dist + F.pad;
+            // Along a ray of direction d the ellipsoid lies within (centre - eye).d -+ |A R^T d|.  For
+            // d = dc that is depth -+ h; a ray at angle <= delta from dc moves the centre term by at
+            // most |depth| delta^2 / 2 + |offset of the centre from the central ray| delta and the
+            // extent by at most amax delta.  The bounding sphere's shell bounds the same range.
+            const float depth = -dot3(O, F.dc);
+            const f3 off = mk3(-O.x - depth * F.dc.x, -O.y - depth * F.dc.y, -O.z - depth * F.dc.z);
+            const float eu = dot3(U, F.dc) * ax.x, ev = dot3(V, F.dc) * ax.y, ew = dot3(W, F.dc) * ax.z;
+            const float ext = sqrtf((eu * eu + ev * ev) + ew * ew) * 1.001f;
+            const float slack = 1.5f * (0.5f * fabsf(depth) * F.delta * F.delta + (sqrtf(dot3(off, off)) + amax) * F.delta) +
+                                1e-5f * dist + F.pad;
+            dmin = fmaxf(dist - rad, depth - ext - slack);
+            dmax = fminf(dist + rad, depth + ext + slack);
             bool ok = p.inv_inter4.w == p.inv_inter4.w; // k is NaN below the density threshold: never hit
             ok = ok && dmax >= F.t0 && dmin <= F.t1;
 #pragma unroll

@@ -165,6 +165,23 @@ int rgx_march_backward(const void *ws, const RgxCamera *cam, const RgxMarch *mar
                        size_t march_ws_bytes, const void *records, size_t records_bytes,
                        RgxStats *stats, void *stream);
 
+/* Replaces the per-tensor `tensor[reordering_index]` gathers of PointCloud.reorder_zordercurve and
+ * OptimizerManager._reorder_tensors (classes/point_cloud.py:1031-1044, classes/optimizer.py:54-66)
+ * by one launch: for each of `count` tensors, dst[i] row j = src[i] row order[j].  src, dst,
+ * row_bytes: HOST arrays of `count` device pointers / row sizes in bytes (multiples of 4); all
+ * tensors have n rows; dst[i] != src[i].  order: device int64, a permutation of 0..n-1. */
+int rgx_gather_rows(int32_t count, const void *const *src, void *const *dst, const int64_t *row_bytes,
+                    const int64_t *order, int64_t n, void *stream);
+
+/* Replaces reduce_supersampling (utils/general_utils.py:489-502) and the clip / 8-bit
+ * quantisation that follow it in the inference loop (scripts/test.py:197-200,
+ * utils/general_utils.py:167): ray_colors ((width*factor_x)*(height*factor_y), 3) as the march
+ * wrote it -> out (height*width, 3), the mean over each pixel's factor_x x factor_y rays, summed in
+ * the reference's order; clipped to [0,1] when clip != 0; out8 = uint8(255 * clipped value).
+ * Either of out, out8 may be NULL. */
+int rgx_reduce_supersampling(const float *ray_colors, int32_t width, int32_t height, int32_t factor_x,
+                             int32_t factor_y, int32_t clip, float *out, uint8_t *out8, void *stream);
+
 /* Test hooks: the two OptiX ray queries on caller-supplied segments (origin = eye,
  * host float[3]; dirs (n,3); tlo/thi (n)).  first-hit: optixTrace SBT offset 0
  * (gaussians_aabb.cu:234-247, 370-380), out_t = smallest hit t or -1.  collect:

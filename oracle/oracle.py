@@ -279,3 +279,17 @@ def render_backward(scene, ctx, ray_colors, dloss):
                densities=g["ddens"], color_features=dsh, sph_gauss_features=dsg,
                bandwidth_sharpness=dsharp, lobe_axis=daxis, rgb=g["drgb"])
     return out, stats
+
+
+def reduce_supersampling(target_width, target_height, ray_colors, factor):
+    """utils/general_utils.py:489-502, restated with the same slicing and summation order."""
+    fx, fy = factor
+    ray_colors = np.asarray(ray_colors, np.float32)
+    s = ray_colors[0::fx].copy()
+    for i in range(1, fx):
+        s += ray_colors[i::fx]
+    s = s.reshape((target_height * fy, target_width, 3))
+    m = s[0::fy].copy()
+    for i in range(1, fy):
+        m += s[i::fy]
+    return m / np.float32(fx * fy)

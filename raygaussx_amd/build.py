@@ -13,7 +13,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librgx.so")
-SOURCES = ["rgx_api.hip", "rgx_build.hip", "rgx_pergauss.hip", "rgx_march.hip"]
+SOURCES = ["rgx_api.hip", "rgx_build.hip", "rgx_pergauss.hip", "rgx_image.hip", "rgx_march.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
          "-munsafe-fp-atomics", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]

@@ -620,3 +620,53 @@ extern "C" int rgx_morton_order(const float *pos, int64_t n, int64_t *codes, int
     }
     return RGX_OK;
 }
+
+// ---------------------------------------------------------------------------
+// Fused multi-tensor gather for the periodic reordering of the point cloud: every
+// per-Gaussian tensor (parameters, Adam moments, statistics) is permuted with the same index
+// (classes/point_cloud.py:1031-1044, classes/optimizer.py:54-66: one `tensor[index]` launch per
+// tensor there).  blockIdx.y picks the tensor; a thread moves one 32-bit word, so writes are
+// coalesced and the reads of a row are contiguous.
+#define RGX_GATHER_MAX 24
+struct GatherArgs {
+    const uint32_t *src[RGX_GATHER_MAX];
+    uint32_t *dst[RGX_GATHER_MAX];
+    int32_t row_words[RGX_GATHER_MAX];
+};
+
+__global__ __launch_bounds__(256) void k_gather_rows(const GatherArgs A, const int64_t *__restrict__ order, int64_t n)
+{
+    const int t = blockIdx.y;
+    const int64_t rw = A.row_words[t];
+    const int64_t total = n * rw;
+    for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t row = e / rw, w = e - row * rw;
+        A.dst[t][e] = A.src[t][order[row] * rw + w];
+    }
+}
+
+extern "C" int rgx_gather_rows(int32_t count, const void *const *src, void *const *dst, const int64_t *row_bytes,
+                               const int64_t *order, int64_t n, void *stream)
+{
+    if (count < 0 || n < 0 || (count > 0 && (!src || !dst || !row_bytes)) || (n > 0 && count > 0 && !order)) return RGX_EINVAL;
+    for (int i = 0; i < count; ++i)
+        if (row_bytes[i] <= 0 || (row_bytes[i] & 3) || row_bytes[i] > 0x7fffffff || ((!src[i] || !dst[i]) && n > 0) || src[i] == dst[i])
+            return RGX_EINVAL;
+    if (n == 0) return RGX_OK;
+    for (int base = 0; base < count; base += RGX_GATHER_MAX) {
+        GatherArgs A;
+        const int m = count - base < RGX_GATHER_MAX ? count - base : RGX_GATHER_MAX;
+        int64_t most = 0;
+        for (int i = 0; i < m; ++i) {
+            A.src[i] = (const uint32_t *)src[base + i];
+            A.dst[i] = (uint32_t *)dst[base + i];
+            A.row_words[i] = (int32_t)(row_bytes[base + i] / 4);
+            most = most > n * A.row_words[i] ? most : n * A.row_words[i];
+        }
+        int64_t blocks = (most + 255) / 256;
+        if (blocks > 65536) blocks = 65536; // grid-stride beyond that
+        hipLaunchKernelGGL(k_gather_rows, dim3((unsigned)blocks, (unsigned)m), dim3(256), 0, (hipStream_t)stream, A, order, n);
+        RGX_LAUNCH_CHECK();
+    }
+    return RGX_OK;
+}

@@ -27,5 +27,27 @@ def morton_order(positions, return_codes=False):
 
 @torch.no_grad()
 def reorder_tensors(order, tensors):
-    """Gather every per-Gaussian tensor (parameters, Adam moments, statistics) with one permutation."""
-    return [None if t is None else t.index_select(0, order) for t in tensors]
+    """Gathers every per-Gaussian tensor (parameters, Adam moments, statistics) with one
+    permutation in one launch: ``[t[order] for t in tensors]`` (``None`` entries pass through).
+    Tensors must have 4- or 8-byte elements (rows that are multiples of 4 bytes)."""
+    order = order.to(torch.int64).contiguous()
+    n = order.shape[0]
+    live = [t for t in tensors if t is not None]
+    if not live:
+        return list(tensors)
+    srcs, dsts = [], []
+    for t in live:
+        if t.shape[0] != n:
+            raise L.RgxError("reorder_tensors: a tensor's first dimension differs from the permutation's length")
+        if not t.is_cuda or (t[0].numel() * t.element_size()) % 4 if n else False:
+            raise L.RgxError("reorder_tensors needs device tensors whose rows are multiples of 4 bytes")
+        srcs.append(t.detach().contiguous())
+        dsts.append(torch.empty_like(srcs[-1]))
+    m = len(srcs)
+    if n:
+        src_p = (C.c_void_p * m)(*[s.data_ptr() for s in srcs])
+        dst_p = (C.c_void_p * m)(*[d.data_ptr() for d in dsts])
+        rows = (C.c_int64 * m)(*[s[0].numel() * s.element_size() for s in srcs])
+        L.check(L.lib().rgx_gather_rows(C.c_int32(m), src_p, dst_p, rows, L.ptr(order), C.c_int64(n), L.stream(order.device)))
+    it = iter(dsts)
+    return [None if t is None else next(it) for t in tensors]

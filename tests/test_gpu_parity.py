@@ -408,6 +408,28 @@ def test_morton_order_bit_exact(gx, orc):
         np.testing.assert_array_equal(order.cpu().numpy(), orc.morton_order(pos))
 
 
+def test_reorder_tensors_is_the_per_tensor_gather(gx):
+    """PointCloud.reorder_zordercurve's gathers (classes/point_cloud.py:1031-1044) in one launch:
+    every tensor equals numpy's `t[index]`, for the parameter shapes of a point cloud with Adam
+    moments (30 tensors: more than one launch holds), ragged sizes and an empty cloud."""
+    from raygaussx_amd.reordering import morton_order, reorder_tensors
+    rng = np.random.default_rng(8)
+    for n in (0, 1, 1000, 100_003):
+        _step(f"reorder_tensors n={n}")
+        shapes = [(n, 3), (n, 3), (n, 4), (n,), (n, 3, 16), (n, 3, 2), (n, 2), (n, 2, 3), (n, 1), (n,)]
+        params = [rng.normal(size=sh).astype(np.float32) for sh in shapes]
+        tensors = params + [p * 2 for p in params] + [p * p for p in params]          # + exp_avg, exp_avg_sq
+        tensors[9] = rng.integers(0, 1 << 40, size=n).astype(np.int64)                # an 8-byte counter
+        order = morton_order(torch.from_numpy(params[0]).to(gx.DEV)) if n else torch.zeros(0, dtype=torch.int64, device=gx.DEV)
+        dev = [torch.from_numpy(t).to(gx.DEV) for t in tensors]
+        dev.insert(3, None)
+        out = reorder_tensors(order, dev)
+        assert out[3] is None and len(out) == len(dev)
+        idx = order.cpu().numpy()
+        for got, src in zip([o for o in out if o is not None], tensors):
+            np.testing.assert_array_equal(got.cpu().numpy(), src[idx])
+
+
 def test_reference_style_inference_loop_reuses_the_tree(gx, orc, c0):
     """scripts/test.py:50-126 pattern: boxes -> one acceleration structure -> several cameras."""
     from raygaussx_amd import optix_utils as u_ox
@@ -432,3 +454,20 @@ def test_reference_style_inference_loop_reuses_the_tree(gx, orc, c0):
         # boxes from the legacy torch routine differ from the canonical ones by rounding, so the scene
         # box (hence texit) may differ in the last ulp; colours still agree to tolerance
         assert np.abs(img.cpu().numpy() - want).max() <= IMG_TOL
+
+
+def test_reduce_supersampling_clip_and_quantise_bit_exact(gx, orc):
+    """The inference loop's image epilogue against the oracle's restatement: floats equal bit for
+    bit (same summation order), clip and uint8(255 x) as numpy computes them."""
+    from raygaussx_amd.general_utils import reduce_supersampling
+    rng = np.random.default_rng(4)
+    for W, H, f in ((33, 21, (1, 1)), (33, 21, (2, 1)), (16, 9, (2, 2)), (5, 7, (3, 2)), (800, 800, (2, 2))):
+        rays = (rng.random((W * f[0] * H * f[1], 3), dtype=np.float32) * 1.4 - 0.2).astype(np.float32)
+        _step(f"reduce_supersampling {W}x{H} x{f}")
+        t = torch.from_numpy(rays).to(gx.DEV)
+        want = orc.reduce_supersampling(W, H, rays, f)
+        got = reduce_supersampling(W, H, t, f).cpu().numpy()
+        np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+        clipped, q = reduce_supersampling(W, H, t, f, clip=True, to_uint8=True)
+        np.testing.assert_array_equal(clipped.cpu().numpy(), want.clip(0, 1))
+        np.testing.assert_array_equal(q.cpu().numpy(), np.uint8(255 * want.clip(0, 1)))

@@ -238,3 +238,18 @@ def test_morton_codes_match_naive_bit_loop(orc):
     two = np.array([[0, 0, 0], [1, 1, 1], [1.0 / 1023 * 1.0001, 0, 0]], np.float32)
     c = orc.morton_codes(two)
     assert c[0] == 0 and c[2] == 1 and c[1] == (1 << 30) - 1
+
+
+def test_reduce_supersampling_is_the_block_mean(orc):
+    """utils/general_utils.py:489-502: each output pixel is the mean of its fx x fy block of rays
+    (checked against a reshape-mean in float64), and factor (1, 1) is the identity."""
+    rng = np.random.default_rng(0)
+    W, H = 7, 5
+    for fx, fy in ((1, 1), (2, 1), (1, 3), (2, 2), (3, 2)):
+        rays = rng.random((W * fx * H * fy, 3), dtype=np.float32)
+        got = orc.reduce_supersampling(W, H, rays, (fx, fy))
+        want = rays.astype(np.float64).reshape(H, fy, W, fx, 3).mean(axis=(1, 3))
+        assert got.shape == (H, W, 3) and got.dtype == np.float32
+        np.testing.assert_allclose(got, want, rtol=0, atol=2e-7)
+        if (fx, fy) == (1, 1):
+            np.testing.assert_array_equal(got.reshape(-1, 3), rays)

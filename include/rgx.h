@@ -165,6 +165,20 @@ int rgx_march_backward(const void *ws, const RgxCamera *cam, const RgxMarch *mar
                        size_t march_ws_bytes, const void *records, size_t records_bytes,
                        RgxStats *stats, void *stream);
 
+/* The interactive viewer's two kernels (its GL window and interop stay with the caller).
+ * rgx_sh_viewer replaces gui_sh (utils/sh_utils.cu:25-119): rgx_sh_forward on tensors that keep
+ * room for max_num_sh coefficients per channel and max_sg_display lobes per Gaussian, of which the
+ * first (degree+1)^2 and g are evaluated.
+ * rgx_march_viewer replaces the viewer's launch of cuda_gui/gaussians_aabb.cu: the forward march on
+ * a black background; frame (W*H uchar4: r, g, b quantised as min(uint(x*256), 255), alpha 255),
+ * depth (W*H): sum over the samples of T (1 - w) t (cuda_gui/gaussians_aabb.cu:189-202).
+ * march->white_background is ignored. */
+int rgx_sh_viewer(const float *eye, const float *pos, const float *sh, const float *sg, const float *sharp,
+                  const float *axis, int32_t g, int32_t degree, int32_t max_num_sh, int32_t max_sg_display,
+                  int64_t n, float *rgb, void *stream);
+int rgx_march_viewer(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
+                     uint8_t *frame, float *depth, void *march_ws, size_t march_ws_bytes, RgxStats *stats, void *stream);
+
 /* Replaces the per-tensor `tensor[reordering_index]` gathers of PointCloud.reorder_zordercurve and
  * OptimizerManager._reorder_tensors (classes/point_cloud.py:1031-1044, classes/optimizer.py:54-66)
  * by one launch: for each of `count` tensors, dst[i] row j = src[i] row order[j].  src, dst,

@@ -220,6 +220,18 @@ def march_trace(cam_struct, march, bmin, bmax, prims, ray, max_slabs=4096, max_i
     return slabs, rgb
 
 
+def march_gui(cam_struct, march, bmin, bmax, prims):
+    """The viewer's launch: (frame (R,4) uint8, expected depth (R,), unquantised colours (R,3))."""
+    prims, bmin, bmax = _f(prims), _f(bmin), _f(bmax)
+    R = cam_struct.width * cam_struct.height
+    frame = np.zeros((R, 4), np.uint8)
+    depth = np.zeros(R, np.float32)
+    colors = np.zeros((R, 3), np.float32)
+    lib().orc_march_gui(C.byref(cam_struct), C.byref(march), _p(bmin), _p(bmax), C.c_int64(prims.shape[0]),
+                        _p(prims), _p(frame), _p(depth), _p(colors))
+    return frame, depth, colors
+
+
 def march_backward(cam_struct, march, bmin, bmax, prims, ray_colors, dloss, ray_ids=None):
     prims, bmin, bmax = _f(prims), _f(bmin), _f(bmax)
     ray_colors, dloss = _f(ray_colors), _f(dloss)

@@ -33,6 +33,8 @@
  *                       empty scene, compositing identity, float64 numpy march
  *   orc_march_backward  torch.autograd through a float64 torch forward with
  *                       frozen hit sets and cut-off masks + central differences
+ *   orc_march_gui       float64 quadrature of int t sigma exp(-tau) dt for one Gaussian,
+ *                       depth / (1 - T) inside the scene box, known quantisation values
  *   orc_morton_codes    naive per-bit loop
  * The reference ships no tests, golden vectors or fixtures for this path, and
  * cannot be built or imported without OptiX/CuPy/an NVIDIA GPU, so there is no
@@ -512,8 +514,13 @@ typedef struct {
 /* a12 + a14: gaussians_aabb.cu:205-340 __raygen__rg and 182-203 colorBlendingT_chunked */
 static void march_forward_ray(const OrcCamera *cam, const OrcMarch *m, const float *bmin,
                               const float *bmax, int64_t N, const float *prims, int64_t ray,
-                              CandList *L, int32_t *ids, float *out_rgb, OrcStats *st, Trace *tr)
+                              CandList *L, int32_t *ids, float *out_rgb, OrcStats *st, Trace *tr,
+                              float *out_depth)
 {
+    /* out_depth (optional): the viewer's expected depth, sum of T (1 - w) t over the samples
+     * (cuda_gui/gaussians_aabb.cu:189-202) */
+    float depth = 0.0f;
+    if (out_depth) *out_depth = 0.0f;
     const unsigned ix = (unsigned)(ray % cam->width), iy = (unsigned)(ray / cam->width);
     const f3 o = mk3(cam->eye[0], cam->eye[1], cam->eye[2]);
     const f3 dir = compute_ray(cam, ix, iy);
@@ -562,6 +569,7 @@ static void march_forward_ray(const OrcCamera *cam, const OrcMarch *m, const flo
             }
             st->slabs++;
             st->hit_pairs += p0;
+            float t_sample = tbuffer + 0.5f * dt; /* cuda_gui/gaussians_aabb.cu:189 */
             for (int base = 0; base < BUFFER_SIZE && T > m->t_eps; base += CHUNK_SIZE) {
                 float local[CHUNK_SIZE][4];
                 accumulate_chunk(prims, ids, p0, tbuffer, dir, dt, base, local);
@@ -571,13 +579,16 @@ static void march_forward_ray(const OrcCamera *cam, const OrcMarch *m, const flo
                     const float s = dt * ((1.0f - w) / fmaxf(x, 1e-6f));
                     const float ts = T * s;
                     C = add3(C, mk3(ts * local[i][1], ts * local[i][2], ts * local[i][3]));
+                    depth += T * (1.0f - w) * t_sample;
                     T *= w;
+                    t_sample += dt;
                 }
             }
         }
         tbuffer += slab_spacing;
     }
     out_rgb[0] = C.x + T * bg; out_rgb[1] = C.y + T * bg; out_rgb[2] = C.z + T * bg;
+    if (out_depth) *out_depth = depth;
 }
 
 static void stats_add(OrcStats *a, const OrcStats *b)
@@ -602,13 +613,46 @@ void orc_march_forward(const OrcCamera *cam, const OrcMarch *m, const float *bmi
 #pragma omp for schedule(dynamic, 16)
         for (int64_t r = 0; r < n; ++r) {
             int64_t ray = ray_ids ? ray_ids[r] : r;
-            march_forward_ray(cam, m, bmin, bmax, N, prims, ray, &L, ids, ray_colors + 3 * ray, &st, NULL);
+            march_forward_ray(cam, m, bmin, bmax, N, prims, ray, &L, ids, ray_colors + 3 * ray, &st, NULL, NULL);
         }
 #pragma omp critical
         stats_add(&total, &st);
         free(ids); free(L.c);
     }
     if (stats) *stats = total;
+}
+
+/* cuda_gui/helpers.h:45-59: clamp to [0,1], then min(uint(x * 256), 255) */
+static unsigned char quantize8(float x)
+{
+    x = fminf(fmaxf(x, 0.0f), 1.0f);
+    const unsigned v = (unsigned)(x * 256.0f);
+    return (unsigned char)(v < 255u ? v : 255u);
+}
+
+/* The viewer's launch (cuda_gui/gaussians_aabb.cu __raygen__rg): the forward march on a black
+ * background, colours quantised to uchar4 (alpha 255), expected depth per ray.  `colors` (W*H,3)
+ * receives the unquantised colours as well. */
+void orc_march_gui(const OrcCamera *cam, const OrcMarch *m, const float *bmin, const float *bmax,
+                   int64_t N, const float *prims, unsigned char *frame, float *depth, float *colors)
+{
+    OrcMarch mm = *m;
+    mm.white_background = 0;
+    const int64_t n = (int64_t)cam->width * cam->height;
+#pragma omp parallel
+    {
+        CandList L = {0, 0, 0};
+        int32_t *ids = (int32_t *)malloc(sizeof(int32_t) * (size_t)(mm.max_prim_slice > 0 ? mm.max_prim_slice : 1));
+        OrcStats st; memset(&st, 0, sizeof st);
+#pragma omp for schedule(dynamic, 16)
+        for (int64_t ray = 0; ray < n; ++ray) {
+            float rgb[3];
+            march_forward_ray(cam, &mm, bmin, bmax, N, prims, ray, &L, ids, rgb, &st, NULL, depth + ray);
+            for (int c = 0; c < 3; ++c) { frame[4 * ray + c] = quantize8(rgb[c]); colors[3 * ray + c] = rgb[c]; }
+            frame[4 * ray + 3] = 255;
+        }
+        free(ids); free(L.c);
+    }
 }
 
 /* One ray with its slab-by-slab hit lists recorded.  Returns the number of
@@ -622,7 +666,7 @@ int orc_march_trace(const OrcCamera *cam, const OrcMarch *m, const float *bmin, 
     OrcStats st; memset(&st, 0, sizeof st);
     Trace tr = {max_slabs, max_ids, 0, 0, slab_t, slab_off, ids_out};
     slab_off[0] = 0;
-    march_forward_ray(cam, m, bmin, bmax, N, prims, ray, &L, ids, rgb_out, &st, &tr);
+    march_forward_ray(cam, m, bmin, bmax, N, prims, ray, &L, ids, rgb_out, &st, &tr, NULL);
     free(ids); free(L.c);
     return tr.n_slabs;
 }

@@ -44,6 +44,8 @@ struct MarchParams {
     const Prim *prims;
     int64_t n;
     float *ray_colors;       // fwd: output
+    uint8_t *frame;          // viewer: uchar4 colours
+    float *depth;            // viewer: expected depth
     const float *fwd_colors; // bwd: forward output (C + T*bg)
     const float *dloss;      // bwd
     float *gbuf;             // bwd: (n,16) gradient block in Morton order
@@ -1179,9 +1181,19 @@ __device__ __forceinline__ void lane_pixel(int px0, int py0, int &px, int &py)
 }
 
 // ---------------------------------------------------------------------------
+// cuda_gui/helpers.h:45-50
+__device__ __forceinline__ uint8_t quantize8(float x)
+{
+    x = fminf(fmaxf(x, 0.0f), 1.0f);
+    const unsigned v = (unsigned)(x * 256.0f);
+    return (uint8_t)(v < 255u ? v : 255u);
+}
+
 // Forward: __raygen__rg (gaussians_aabb.cu:205-340), accumulateChunk (112-180),
-// colorBlendingT_chunked (182-203).
-template <bool RECORD>
+// colorBlendingT_chunked (182-203).  VIEWER: the interactive viewer's variant of the same march
+// (cuda_gui/gaussians_aabb.cu): black background, uchar4 colours, and the expected depth
+// sum T (1 - w) t over the samples (its colorBlendingT_chunked, 183-205).
+template <bool RECORD, bool VIEWER>
 __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchParams P)
 {
     RGX_TILE_LDS();
@@ -1198,7 +1210,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
     RayState R;
     ray_begin<false>(P, px, py, valid, R);
     const f3 dir = R.dir;
-    float Cr = 0.f, Cg = 0.f, Cb = 0.f;
+    float Cr = 0.f, Cg = 0.f, Cb = 0.f, depth = 0.f;
     Window Wn = {0.f, 0, false, 4, false};
 
     while (__any(R.active)) {
@@ -1213,6 +1225,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
 #pragma unroll
             for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
             f3 rdt = dir * fmaf(dt, 0.5f, R.tbuffer); // samples 0..15
+            float t_sample = R.tbuffer + 0.5f * dt;
             auto accumulate = [&](const auto &e, bool hit, bool, auto) {
                 if (hit) {
                     const float4 col = e.prim->rgba4;
@@ -1243,6 +1256,10 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
                     Cr = fmaf(ts, cr[i], Cr);
                     Cg = fmaf(ts, cg[i], Cg);
                     Cb = fmaf(ts, cb[i], Cb);
+                    if constexpr (VIEWER) {
+                        depth += R.T * (1.0f - w) * t_sample;
+                        t_sample += dt;
+                    }
                     R.T *= w;
                 }
             };
@@ -1267,11 +1284,16 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
         slab_end(R, need, p0, found, searched_to, cn);
     }
     if (valid) {
-        const float bg = P.m.white_background ? 1.0f : 0.0f;
         const int64_t ray = (int64_t)py * P.cam.width + px;
-        P.ray_colors[3 * ray] = Cr + R.T * bg;
-        P.ray_colors[3 * ray + 1] = Cg + R.T * bg;
-        P.ray_colors[3 * ray + 2] = Cb + R.T * bg;
+        if constexpr (VIEWER) {
+            *(uchar4 *)(P.frame + 4 * ray) = make_uchar4(quantize8(Cr), quantize8(Cg), quantize8(Cb), 255);
+            P.depth[ray] = depth;
+        } else {
+            const float bg = P.m.white_background ? 1.0f : 0.0f;
+            P.ray_colors[3 * ray] = Cr + R.T * bg;
+            P.ray_colors[3 * ray + 1] = Cg + R.T * bg;
+            P.ray_colors[3 * ray + 2] = Cb + R.T * bg;
+        }
     }
     rec.finish();
     flush_stats(P.stats, cn);
@@ -1671,6 +1693,8 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     P.prims = (const Prim *)prims;
     P.n = n;
     P.ray_colors = nullptr;
+    P.frame = nullptr;
+    P.depth = nullptr;
     P.fwd_colors = nullptr;
     P.dloss = nullptr;
     P.gbuf = (float *)((char *)march_ws + M.gbuf);
@@ -1721,8 +1745,24 @@ extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const Rgx
     if (rc) return rc;
     P.ray_colors = ray_colors;
     void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
-    if (P.records) hipLaunchKernelGGL(k_march_fwd<true>, march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
-    else hipLaunchKernelGGL(k_march_fwd<false>, march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    if (P.records) hipLaunchKernelGGL((k_march_fwd<true, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    else hipLaunchKernelGGL((k_march_fwd<false, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    rgx_span_end(span, (hipStream_t)stream);
+    RGX_LAUNCH_CHECK();
+    return RGX_OK;
+}
+
+extern "C" int rgx_march_viewer(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
+                                uint8_t *frame, float *depth, void *march_ws, size_t march_ws_bytes, RgxStats *stats, void *stream)
+{
+    MarchParams P;
+    const int rc = fill_params(P, ws, cam, march, prims, n, march_ws, march_ws_bytes, stats);
+    if (rc != RGX_OK) return rc;
+    if (!frame || !depth || ((uintptr_t)frame & 3u)) return RGX_EINVAL;
+    P.frame = frame;
+    P.depth = depth;
+    void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
+    hipLaunchKernelGGL((k_march_fwd<false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     rgx_span_end(span, (hipStream_t)stream);
     RGX_LAUNCH_CHECK();
     return RGX_OK;

@@ -39,8 +39,12 @@ __device__ __forceinline__ void sh_basis(float x, float y, float z, float *b)
 template <int DEG>
 __global__ __launch_bounds__(256) void k_sh_fwd(f3 eye, const float *__restrict__ pos, const float *__restrict__ sh,
                                                 const float *__restrict__ sg, const float *__restrict__ sharp,
-                                                const float *__restrict__ axis, int G, int64_t n, float *__restrict__ rgb)
+                                                const float *__restrict__ axis, int G, int Gs, int Ks, int64_t n,
+                                                float *__restrict__ rgb)
 {
+    // Gs, Ks: lobes / coefficients STORED per Gaussian and channel (>= G, >= K): the viewer keeps
+    // room for the largest model and evaluates the first G lobes and K coefficients (gui_sh,
+    // sh_utils.cu:25-119); everywhere else they equal G and K.
     constexpr int K = (DEG + 1) * (DEG + 1);
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
@@ -49,14 +53,14 @@ __global__ __launch_bounds__(256) void k_sh_fwd(f3 eye, const float *__restrict_
     const f3 d = mk3(v.x / len, v.y / len, v.z / len);
     float res[3] = {0.f, 0.f, 0.f};
     for (int l = 0; l < G; ++l) {
-        const f3 ax = mk3(axis[(i * G + l) * 3], axis[(i * G + l) * 3 + 1], axis[(i * G + l) * 3 + 2]);
-        const float g = expf(sharp[i * G + l] * (dot3(d, ax) - 1.0f));
-        for (int c = 0; c < 3; ++c) res[c] += sg[i * G * 3 + c * G + l] * g;
+        const f3 ax = mk3(axis[(i * Gs + l) * 3], axis[(i * Gs + l) * 3 + 1], axis[(i * Gs + l) * 3 + 2]);
+        const float g = expf(sharp[i * Gs + l] * (dot3(d, ax) - 1.0f));
+        for (int c = 0; c < 3; ++c) res[c] += sg[i * Gs * 3 + c * Gs + l] * g;
     }
     float b[K];
     sh_basis<DEG>(d.x, d.y, d.z, b);
     for (int c = 0; c < 3; ++c) {
-        const float *s = sh + (i * 3 + c) * K;
+        const float *s = sh + (i * 3 + c) * Ks;
         float r = res[c];
 #pragma unroll
         for (int j = 0; j < K; ++j) r += b[j] * s[j];
@@ -163,11 +167,12 @@ __global__ __launch_bounds__(256) void k_pack(f3 eye, const float *__restrict__ 
 
 static inline dim3 grid_for(int64_t n, int block) { return dim3((unsigned)((n + block - 1) / block)); }
 
-extern "C" int rgx_sh_forward(const float *eye, const float *pos, const float *sh, const float *sg, const float *sharp,
-                              const float *axis, int32_t g, int32_t degree, int64_t n, float *rgb, void *stream)
+static int sh_forward_launch(const float *eye, const float *pos, const float *sh, const float *sg, const float *sharp,
+                             const float *axis, int32_t g, int32_t degree, int32_t gs, int32_t ks, int64_t n, float *rgb,
+                             void *stream)
 {
-    if (!eye || n < 0 || degree < 0 || degree > 3 || g < 0 || (n > 0 && (!pos || !sh || !rgb)) ||
-        (g > 0 && n > 0 && (!sg || !sharp || !axis)))
+    if (!eye || n < 0 || degree < 0 || degree > 3 || g < 0 || gs < g || ks < (degree + 1) * (degree + 1) ||
+        (n > 0 && (!pos || !sh || !rgb)) || (g > 0 && n > 0 && (!sg || !sharp || !axis)))
         return RGX_EINVAL;
     if (n == 0) return RGX_OK;
     hipStream_t s = (hipStream_t)stream;
@@ -175,14 +180,27 @@ extern "C" int rgx_sh_forward(const float *eye, const float *pos, const float *s
     const dim3 grid = grid_for(n, 256), block(256);
     void *span = rgx_span_begin(RGX_T_SH_FWD, s);
     switch (degree) {
-    case 0: hipLaunchKernelGGL(k_sh_fwd<0>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, n, rgb); break;
-    case 1: hipLaunchKernelGGL(k_sh_fwd<1>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, n, rgb); break;
-    case 2: hipLaunchKernelGGL(k_sh_fwd<2>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, n, rgb); break;
-    default: hipLaunchKernelGGL(k_sh_fwd<3>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, n, rgb); break;
+    case 0: hipLaunchKernelGGL(k_sh_fwd<0>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, gs, ks, n, rgb); break;
+    case 1: hipLaunchKernelGGL(k_sh_fwd<1>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, gs, ks, n, rgb); break;
+    case 2: hipLaunchKernelGGL(k_sh_fwd<2>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, gs, ks, n, rgb); break;
+    default: hipLaunchKernelGGL(k_sh_fwd<3>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, gs, ks, n, rgb); break;
     }
     rgx_span_end(span, s);
     RGX_LAUNCH_CHECK();
     return RGX_OK;
+}
+
+extern "C" int rgx_sh_forward(const float *eye, const float *pos, const float *sh, const float *sg, const float *sharp,
+                              const float *axis, int32_t g, int32_t degree, int64_t n, float *rgb, void *stream)
+{
+    return sh_forward_launch(eye, pos, sh, sg, sharp, axis, g, degree, g, (degree + 1) * (degree + 1), n, rgb, stream);
+}
+
+extern "C" int rgx_sh_viewer(const float *eye, const float *pos, const float *sh, const float *sg, const float *sharp,
+                             const float *axis, int32_t g, int32_t degree, int32_t max_num_sh, int32_t max_sg_display,
+                             int64_t n, float *rgb, void *stream)
+{
+    return sh_forward_launch(eye, pos, sh, sg, sharp, axis, g, degree, max_sg_display, max_num_sh, n, rgb, stream);
 }
 
 extern "C" int rgx_sh_backward(const float *eye, const float *pos, const float *sh, const float *sg, const float *sharp,

@@ -207,6 +207,33 @@ def march_forward(gas, cam, prims, dt_step, dynamic_sampling, max_prim_slice, wh
     return ray_colors
 
 
+def march_viewer(gas, cam, prims, dt_step, dynamic_sampling, max_prim_slice, t_eps=TRANSMITTANCE_EPSILON, stats=None):
+    """The interactive viewer's launch (cuda_gui/gaussians_aabb.cu): ``(frame (H, W, 4) uint8, depth (H, W))``,
+    black background, colours quantised as the viewer does, expected depth per ray."""
+    n, dev = prims.shape[0], prims.device
+    m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), 0, t_eps)
+    ws = _march_ws(n, cam.width * cam.height, max_prim_slice, dev)
+    frame = torch.empty(cam.height, cam.width, 4, dtype=torch.uint8, device=dev)
+    depth = torch.empty(cam.height, cam.width, dtype=torch.float32, device=dev)
+    L.check(L.lib().rgx_march_viewer(L.ptr(gas.ws), C.byref(cam), C.byref(m), L.ptr(prims), C.c_int64(n), L.ptr(frame),
+                                     L.ptr(depth), L.ptr(ws), C.c_size_t(ws.numel()), L.ptr(stats), L.stream(dev)))
+    return frame, depth
+
+
+def sh_viewer(camera_center, positions, sh, sph_gauss_features, bandwidth_sharpness, lobe_axis, num_sph_gauss,
+              sh_degree, max_num_sh, max_sg_display):
+    """gui_sh (utils/sh_utils.cu:25-119): per-Gaussian colour from tensors that keep room for ``max_num_sh``
+    coefficients per channel and ``max_sg_display`` lobes, evaluating the first ``(sh_degree+1)^2`` and
+    ``num_sph_gauss`` of them."""
+    n = positions.shape[0]
+    rgb = torch.empty(n, 3, dtype=torch.float32, device=positions.device)
+    L.check(L.lib().rgx_sh_viewer(L.host3(camera_center), L.ptr(L.f32(positions)), L.ptr(L.f32(sh)),
+                                  L.ptr(sph_gauss_features), L.ptr(bandwidth_sharpness), L.ptr(lobe_axis),
+                                  C.c_int32(num_sph_gauss), C.c_int32(sh_degree), C.c_int32(max_num_sh),
+                                  C.c_int32(max_sg_display), C.c_int64(n), L.ptr(rgb), L.stream(positions.device)))
+    return rgb
+
+
 def march_backward(gas, cam, prims, ray_colors, dloss, dt_step, dynamic_sampling, max_prim_slice,
                    white_background=True, t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None):
     n, dev = prims.shape[0], prims.device

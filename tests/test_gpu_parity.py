@@ -471,3 +471,46 @@ def test_reduce_supersampling_clip_and_quantise_bit_exact(gx, orc):
         clipped, q = reduce_supersampling(W, H, t, f, clip=True, to_uint8=True)
         np.testing.assert_array_equal(clipped.cpu().numpy(), want.clip(0, 1))
         np.testing.assert_array_equal(q.cpu().numpy(), np.uint8(255 * want.clip(0, 1)))
+
+
+def test_viewer_frame_depth_and_strided_colours(gx, orc, c0):
+    """The interactive viewer's two kernels: the march with uchar4 colours and expected depth
+    (cuda_gui/gaussians_aabb.cu) against the oracle's restatement, and gui_sh's strided tensors
+    against the plain colour evaluation of the coefficients and lobes it selects."""
+    from raygaussx_amd import optix_utils as u_ox
+    sc, cam, cfg = c0
+    sc = dict(sc)
+    sc["scales"] = sc["scales"] * 2.0
+    img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], False, cfg["max_prim_slice"], white_background=False)
+    frame, depth, colors = orc.march_gui(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"])
+    d = gx.to_dev(sc)
+    gas = u_ox.AccelerationStructure(4096, gx.DEV).build_from_gaussians(d["positions"], d["scales"], d["quaternions"],
+                                                                         d["densities"])
+    ps = u_ox.pack_prims(gas, ctx["eye"], d["positions"], d["scales"], d["quaternions"], d["densities"],
+                         torch.from_numpy(ctx["rgb"]).to(gx.DEV))
+    _step("viewer march")
+    f_gpu, z_gpu = u_ox.march_viewer(gas, u_ox.camera_struct(cam), ps, cfg["dt_step"], False, cfg["max_prim_slice"])
+    f_gpu, z_gpu = f_gpu.cpu().numpy().reshape(-1, 4), z_gpu.cpu().numpy().reshape(-1)
+    assert (depth > 0).sum() > 5000
+    assert np.abs(z_gpu - depth).max() <= 1e-4 * depth.max()
+    np.testing.assert_array_equal(z_gpu == 0, depth == 0)
+    # colours agree to 1e-4, so a quantised channel may differ by one step where it sits on a boundary
+    diff = np.abs(f_gpu.astype(np.int32) - frame.astype(np.int32))
+    assert diff.max() <= 1 and (diff > 0).mean() < 0.02 and (f_gpu[:, 3] == 255).all()
+    _step("viewer colours")
+    rng = np.random.default_rng(6)
+    n, kmax, gmax = 3000, 16, 4
+    pos = rng.normal(size=(n, 3)).astype(np.float32)
+    sh = (rng.normal(size=(n, 3, kmax)) * 0.2).astype(np.float32)
+    sg = (rng.normal(size=(n, 3, gmax)) * 0.1).astype(np.float32)
+    sharp = rng.uniform(0.5, 3, size=(n, gmax)).astype(np.float32)
+    ax = rng.normal(size=(n, gmax, 3)).astype(np.float32)
+    ax /= np.linalg.norm(ax, axis=2, keepdims=True)
+    eye = np.array([0.3, -4.0, 1.0], np.float32)
+    for deg, g in ((0, 0), (1, 2), (2, 4), (3, 1)):
+        k = (deg + 1) ** 2
+        want = orc.sh_forward(eye, pos, np.ascontiguousarray(sh[:, :, :k]),
+                              *((np.ascontiguousarray(sg[:, :, :g]), np.ascontiguousarray(sharp[:, :g]),
+                                 np.ascontiguousarray(ax[:, :g])) if g else (None, None, None)))
+        got = u_ox.sh_viewer(eye, *[torch.from_numpy(a).to(gx.DEV) for a in (pos, sh, sg, sharp, ax)], g, deg, kmax, gmax)
+        np.testing.assert_allclose(got.cpu().numpy(), want, rtol=2e-5, atol=2e-6)

@@ -243,3 +243,56 @@ def test_backward_matches_central_differences_through_whole_operator(orc):
     ana = g["color_features"][:, 1, 0]
     cos, rel = _cos_rel(ana, num)
     assert cos > 0.999 and rel < 3e-2, (cos, rel)
+
+
+def test_viewer_depth_and_quantised_colours(orc):
+    """The viewer's outputs (cuda_gui/gaussians_aabb.cu): expected depth sum T (1 - w) t and
+    uchar4 colours on a black background.  (i) One isotropic Gaussian on the ray axis against a
+    float64 quadrature of int t sigma(t) exp(-tau(t)) dt with the truncated density; (ii) with
+    colour 1 the image is 1 - T, so depth / colour is a weighted mean distance that must lie inside
+    the Gaussian; (iii) in a scene, depth / (1 - T) lies between the box entry and exit and the
+    frame is the colours' quantisation, with the known values 0 -> 0, 0.5 -> 128, 1 -> 255."""
+    rho, s, dist = 3.0, 0.05, 4.0
+    k = math.sqrt(2 * math.log(rho / 0.1))
+    cam = _axis_camera(dist=dist)
+    centre = 4 * 9 + 4
+    sc = _one_gaussian(rho, s, (1.0, 1.0, 1.0))
+    t = np.linspace(dist - k * s, dist + k * s, 400001)
+    sigma = rho * np.exp(-0.5 * ((t - dist) / s) ** 2)
+    tau = np.concatenate([[0.0], np.cumsum(0.5 * (sigma[1:] + sigma[:-1]) * np.diff(t))])
+    f = t * sigma * np.exp(-tau)
+    want_depth = float(np.sum(0.5 * (f[1:] + f[:-1]) * np.diff(t)))
+    want_alpha = 1.0 - math.exp(-tau[-1])
+    for dt in (0.002, 0.001):
+        _, _, ctx = _render(orc, sc, cam, dt, white=False)
+        frame, depth, colors = orc.march_gui(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"])
+        assert abs(colors[centre, 0] - want_alpha) < 0.1 * dt + 1e-5
+        # depth carries the same O(dt) truncation-boundary error as the optical depth, times t
+        assert abs(depth[centre] - want_depth) < dist * (0.1 * dt + 1e-5) + dt * want_alpha
+        mean_t = depth[centre] / colors[centre, 0]
+        assert dist - k * s < mean_t < dist            # absorption weights the near side
+        assert depth[0] == 0.0 and (frame[0] == (0, 0, 0, 255)).all()      # a ray that misses
+    # (iii) a scene
+    scn = scenes.scene_to_numpy(scenes.make_scene(0, n=800, sh_degree=0, seed=5))
+    scn["scales"] = scn["scales"] * 2.5
+    scn["color_features"][:] = (1.0 - 0.5) / 0.28209479177387814          # colour exactly 1
+    cam2 = scenes.make_camera(0, 0, width=32, height=32)
+    img, st, ctx = _render(orc, scn, cam2, 0.0025, cap=800, white=False)
+    frame, depth, colors = orc.march_gui(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"])
+    np.testing.assert_array_equal(colors, img)                            # same march as the forward
+    hit = colors[:, 0] > 1e-3
+    assert hit.sum() > 300
+    eye = cam2.camera_center.numpy().astype(np.float64)
+    dirs = orc.ray_dirs(ctx["cs"], np.arange(32 * 32)).astype(np.float64)
+    lo = (ctx["bmin"].astype(np.float64) - eye) / dirs
+    hi = (ctx["bmax"].astype(np.float64) - eye) / dirs
+    tenter = np.minimum(lo, hi).max(1)
+    texit = np.maximum(lo, hi).min(1)
+    mean_t = depth[hit] / colors[hit, 0]
+    assert (mean_t > tenter[hit] - 1e-3).all() and (mean_t < texit[hit] + 1e-3).all()
+    np.testing.assert_array_equal(frame[:, :3], np.minimum(np.floor(np.clip(colors, 0, 1) * 256.0), 255).astype(np.uint8))
+    assert (frame[:, 3] == 255).all()
+    one = _one_gaussian(60.0, 0.2, (0.5, 1.0, 0.0))                       # opaque: colours reach (0.5, 1, 0)
+    _, _, ctx1 = _render(orc, one, cam, 0.002, white=False)
+    f1, _, c1 = orc.march_gui(ctx1["cs"], ctx1["ms"], ctx1["bmin"], ctx1["bmax"], ctx1["prims"])
+    assert abs(c1[centre, 1] - 1.0) < 2e-3 and f1[centre, 2] == 0 and f1[centre, 1] >= 254 and 127 <= f1[centre, 0] <= 128

@@ -187,6 +187,13 @@ int rgx_march_viewer(const void *ws, const RgxCamera *cam, const RgxMarch *march
 int rgx_gather_rows(int32_t count, const void *const *src, void *const *dst, const int64_t *row_bytes,
                     const int64_t *order, int64_t n, void *stream);
 
+/* Replaces distCUDA2 of the simple-knn extension (submodules/simple-knn/simple_knn.cu:186-222,
+ * called at classes/point_cloud.py:252 to initialise the scales): mean_dist2[i] = mean of the
+ * squared distances from point i to its three nearest other points (FLT_MAX stands in for a
+ * missing neighbour when n < 4, as there).  pos (n,3).  ws from rgx_knn_workspace_bytes. */
+int rgx_knn_workspace_bytes(int64_t n, size_t *bytes);
+int rgx_dist2_knn3(const float *pos, int64_t n, float *mean_dist2, void *ws, size_t ws_bytes, void *stream);
+
 /* Replaces reduce_supersampling (utils/general_utils.py:489-502) and the clip / 8-bit
  * quantisation that follow it in the inference loop (scripts/test.py:197-200,
  * utils/general_utils.py:167): ray_colors ((width*factor_x)*(height*factor_y), 3) as the march

@@ -293,6 +293,14 @@ def render_backward(scene, ctx, ray_colors, dloss):
     return out, stats
 
 
+def dist2_knn3(pos):
+    """distCUDA2: mean squared distance to the three nearest other points (brute force)."""
+    pos = _f(pos)
+    out = np.empty(pos.shape[0], np.float32)
+    lib().orc_dist2_knn3(C.c_int64(pos.shape[0]), _p(pos), _p(out))
+    return out
+
+
 def reduce_supersampling(target_width, target_height, ray_colors, factor):
     """utils/general_utils.py:489-502, restated with the same slicing and summation order."""
     fx, fy = factor

@@ -36,10 +36,12 @@
  *   orc_march_gui       float64 quadrature of int t sigma exp(-tau) dt for one Gaussian,
  *                       depth / (1 - T) inside the scene box, known quantisation values
  *   orc_morton_codes    naive per-bit loop
+ *   orc_dist2_knn3      scipy.spatial.cKDTree (k = 4 with the point itself) in float64
  * The reference ships no tests, golden vectors or fixtures for this path, and
  * cannot be built or imported without OptiX/CuPy/an NVIDIA GPU, so there is no
  * oracle/_ref build.
  */
+#include <float.h>
 #include <math.h>
 #include <stdint.h>
 #include <stdlib.h>
@@ -950,4 +952,25 @@ void orc_set_num_threads(int n)
 #else
     (void)n;
 #endif
+}
+
+/* ------------------------------------------------------------------------- */
+/* distCUDA2 (submodules/simple-knn/simple_knn.cu:137-184): mean of the squared
+ * distances to the three nearest other points.  The reference prunes with Morton-sorted boxes;
+ * its pruning is exact, so brute force gives the same three distances.  updateKBest<3> is kept
+ * as written (insertion into a sorted triple); dist = (dx*dx + dy*dy) + dz*dz. */
+void orc_dist2_knn3(int64_t n, const float *pos, float *out)
+{
+#pragma omp parallel for schedule(dynamic, 64)
+    for (int64_t i = 0; i < n; ++i) {
+        float best[3] = {FLT_MAX, FLT_MAX, FLT_MAX};
+        for (int64_t j = 0; j < n; ++j) {
+            if (j == i) continue;
+            const float dx = pos[3 * j] - pos[3 * i], dy = pos[3 * j + 1] - pos[3 * i + 1], dz = pos[3 * j + 2] - pos[3 * i + 2];
+            float dist = (dx * dx + dy * dy) + dz * dz;
+            for (int k = 0; k < 3; ++k)
+                if (best[k] > dist) { const float t = best[k]; best[k] = dist; dist = t; }
+        }
+        out[i] = ((best[0] + best[1]) + best[2]) / 3.0f;
+    }
 }

@@ -4,6 +4,7 @@
 // and the AABB pass feeding it (optix_utils.py:36-109).  Also hosts the 30-bit
 // Morton ordering of the point cloud (utils/reordering_utils.py:55-104).
 #include "rgx_device.h"
+#include <float.h>
 
 // ---------------------------------------------------------------------------
 // order-preserving float <-> int encoding for atomicMin/atomicMax
@@ -668,5 +669,159 @@ extern "C" int rgx_gather_rows(int32_t count, const void *const *src, void *cons
         hipLaunchKernelGGL(k_gather_rows, dim3((unsigned)blocks, (unsigned)m), dim3(256), 0, (hipStream_t)stream, A, order, n);
         RGX_LAUNCH_CHECK();
     }
+    return RGX_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Mean squared distance of every point to its three nearest neighbours: distCUDA2 of the
+// simple-knn extension (submodules/simple-knn/simple_knn.cu:186-222; used to initialise the scales,
+// classes/point_cloud.py:252).  As there: points sorted along a Morton curve, boxes of consecutive
+// sorted points, every point scans the boxes that can still hold one of its three nearest (the
+// pruning is exact, so the result is the exact 3-NN mean whatever the order and the box size).
+// Here the boxes have two levels (256 points, 64 boxes) so that a point looks at a few hundred box
+// bounds instead of all n / 256, and the sorted points are gathered once so that the scans read
+// consecutive memory.  Distances are (dx*dx + dy*dy) + dz*dz without contraction.
+#define RGX_KNN_BOX 256
+#define RGX_KNN_SUPER 64
+
+__global__ __launch_bounds__(256) void k_knn_gather(const float *__restrict__ pos, const uint32_t *__restrict__ order, int64_t n,
+                                                    float4 *__restrict__ pts)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t j = order[i];
+    pts[i] = make_float4(pos[3 * j], pos[3 * j + 1], pos[3 * j + 2], 0.f);
+}
+
+// bounds of `per` consecutive items: points (float4) at level 0, boxes (lo, hi pairs) above
+__global__ __launch_bounds__(256) void k_knn_bounds(const float4 *__restrict__ lo_in, const float4 *__restrict__ hi_in,
+                                                    int stride, int64_t n_in, int per, float4 *__restrict__ out)
+{
+    const int64_t b = blockIdx.x;
+    float mn[3] = {INFINITY, INFINITY, INFINITY}, mx[3] = {-INFINITY, -INFINITY, -INFINITY};
+    for (int64_t i = b * per + threadIdx.x; i < n_in && i < (b + 1) * per; i += blockDim.x) {
+        const float4 l = lo_in[i * stride], h = hi_in[i * stride];
+        mn[0] = fminf(mn[0], l.x); mn[1] = fminf(mn[1], l.y); mn[2] = fminf(mn[2], l.z);
+        mx[0] = fmaxf(mx[0], h.x); mx[1] = fmaxf(mx[1], h.y); mx[2] = fmaxf(mx[2], h.z);
+    }
+    __shared__ float red[4][6];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int a = 0; a < 3; ++a) {
+        const float l = wave_min(mn[a]), h = wave_max(mx[a]);
+        if (lane == 0) { red[wave][a] = l; red[wave][a + 3] = h; }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int a = 0; a < 6; ++a)
+            for (int w = 1; w < 4; ++w) red[0][a] = a < 3 ? fminf(red[0][a], red[w][a]) : fmaxf(red[0][a], red[w][a]);
+        out[2 * b] = make_float4(red[0][0], red[0][1], red[0][2], 0.f);
+        out[2 * b + 1] = make_float4(red[0][3], red[0][4], red[0][5], 0.f);
+    }
+}
+
+// simple_knn.cu:124-135 distBoxPoint
+__device__ __forceinline__ float knn_box_dist(float4 lo, float4 hi, float4 p)
+{
+    float dx = 0.f, dy = 0.f, dz = 0.f;
+    if (p.x < lo.x || p.x > hi.x) dx = fminf(fabsf(p.x - lo.x), fabsf(p.x - hi.x));
+    if (p.y < lo.y || p.y > hi.y) dy = fminf(fabsf(p.y - lo.y), fabsf(p.y - hi.y));
+    if (p.z < lo.z || p.z > hi.z) dz = fminf(fabsf(p.z - lo.z), fabsf(p.z - hi.z));
+    return (dx * dx + dy * dy) + dz * dz;
+}
+
+// simple_knn.cu:137-151 updateKBest<3>
+__device__ __forceinline__ void knn_update(float4 ref, float4 q, float *best)
+{
+    const float dx = q.x - ref.x, dy = q.y - ref.y, dz = q.z - ref.z;
+    float dist = (dx * dx + dy * dy) + dz * dz;
+#pragma unroll
+    for (int j = 0; j < 3; ++j)
+        if (best[j] > dist) {
+            const float t = best[j];
+            best[j] = dist;
+            dist = t;
+        }
+}
+
+// simple_knn.cu:153-184 boxMeanDist
+__global__ __launch_bounds__(256) void k_knn3(const float4 *__restrict__ pts, const uint32_t *__restrict__ order, int64_t n,
+                                              const float4 *__restrict__ boxes, int64_t nb, const float4 *__restrict__ supers,
+                                              int64_t ns, float *__restrict__ out)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float4 p = pts[i];
+    float best[3] = {FLT_MAX, FLT_MAX, FLT_MAX};
+    for (int64_t j = i - 3 < 0 ? 0 : i - 3; j <= (i + 3 > n - 1 ? n - 1 : i + 3); ++j)
+        if (j != i) knn_update(p, pts[j], best);
+    const float reject = best[2];
+    best[0] = best[1] = best[2] = FLT_MAX;
+    for (int64_t s = 0; s < ns; ++s) {
+        const float ds = knn_box_dist(supers[2 * s], supers[2 * s + 1], p);
+        if (ds > reject || ds > best[2]) continue;
+        const int64_t b1 = (s + 1) * RGX_KNN_SUPER < nb ? (s + 1) * RGX_KNN_SUPER : nb;
+        for (int64_t b = s * RGX_KNN_SUPER; b < b1; ++b) {
+            const float d = knn_box_dist(boxes[2 * b], boxes[2 * b + 1], p);
+            if (d > reject || d > best[2]) continue;
+            const int64_t j1 = (b + 1) * RGX_KNN_BOX < n ? (b + 1) * RGX_KNN_BOX : n;
+            for (int64_t j = b * RGX_KNN_BOX; j < j1; ++j)
+                if (j != i) knn_update(p, pts[j], best);
+        }
+    }
+    out[order[i]] = ((best[0] + best[1]) + best[2]) / 3.0f;
+}
+
+struct KnnLayout {
+    MortonLayout m;
+    size_t pts, boxes, supers, total;
+    int64_t nb, ns;
+};
+static inline KnnLayout knn_layout(int64_t n)
+{
+    KnnLayout K;
+    K.m = morton_layout(n);
+    const size_t nn = (size_t)(n > 0 ? n : 1);
+    K.nb = (int64_t)((nn + RGX_KNN_BOX - 1) / RGX_KNN_BOX);
+    K.ns = (K.nb + RGX_KNN_SUPER - 1) / RGX_KNN_SUPER;
+    size_t off = K.m.total;
+    K.pts = off;    off = rgx_align_up(off + nn * 16, 256);
+    K.boxes = off;  off = rgx_align_up(off + (size_t)K.nb * 32, 256);
+    K.supers = off; off = rgx_align_up(off + (size_t)K.ns * 32, 256);
+    K.total = off;
+    return K;
+}
+
+extern "C" int rgx_knn_workspace_bytes(int64_t n, size_t *bytes)
+{
+    if (n < 0 || !bytes || n > 0x3fffffff) return RGX_EINVAL;
+    *bytes = knn_layout(n).total;
+    return RGX_OK;
+}
+
+extern "C" int rgx_dist2_knn3(const float *pos, int64_t n, float *mean_dist2, void *ws, size_t ws_bytes, void *stream)
+{
+    if (n < 0 || n > 0x3fffffff || !ws || (n > 0 && (!pos || !mean_dist2))) return RGX_EINVAL;
+    const KnnLayout K = knn_layout(n);
+    if (ws_bytes < K.total || ((uintptr_t)ws & 255u)) return RGX_EWORKSPACE;
+    if (n == 0) return RGX_OK;
+    hipStream_t s = (hipStream_t)stream;
+    char *w = (char *)ws;
+    int32_t *mn = (int32_t *)(w + K.m.enc), *mx = mn + 4;
+    uint32_t *k0 = (uint32_t *)(w + K.m.keys0), *k1 = (uint32_t *)(w + K.m.keys1);
+    uint32_t *v0 = (uint32_t *)(w + K.m.vals0), *v1 = (uint32_t *)(w + K.m.vals1);
+    float4 *pts = (float4 *)(w + K.pts), *boxes = (float4 *)(w + K.boxes), *supers = (float4 *)(w + K.supers);
+    hipLaunchKernelGGL(k_init_enc, dim3(1), dim3(64), 0, s, mn, mx);
+    hipLaunchKernelGGL(k_pos_minmax, grid_for(n, 256), dim3(256), 0, s, pos, n, mn, mx);
+    hipLaunchKernelGGL(k_decode_enc, dim3(1), dim3(64), 0, s, mn, mx);
+    hipLaunchKernelGGL(k_morton30, grid_for(n, 256), dim3(256), 0, s, pos, n, (const float *)mn, (const float *)mx, k0, v0,
+                       (int64_t *)nullptr);
+    RGX_LAUNCH_CHECK();
+    const int r = radix_sort<uint32_t>(k0, v0, k1, v1, n, 32, (uint32_t *)(w + K.m.hist), s);
+    if (r < 0) return r;
+    hipLaunchKernelGGL(k_knn_gather, grid_for(n, 256), dim3(256), 0, s, pos, v0, n, pts);
+    hipLaunchKernelGGL(k_knn_bounds, dim3((unsigned)K.nb), dim3(256), 0, s, pts, pts, 1, n, RGX_KNN_BOX, boxes);
+    hipLaunchKernelGGL(k_knn_bounds, dim3((unsigned)K.ns), dim3(256), 0, s, boxes, boxes + 1, 2, K.nb, RGX_KNN_SUPER, supers);
+    hipLaunchKernelGGL(k_knn3, grid_for(n, 256), dim3(256), 0, s, pts, v0, n, boxes, K.nb, supers, K.ns, mean_dist2);
+    RGX_LAUNCH_CHECK();
     return RGX_OK;
 }

@@ -514,3 +514,26 @@ def test_viewer_frame_depth_and_strided_colours(gx, orc, c0):
                                  np.ascontiguousarray(ax[:, :g])) if g else (None, None, None)))
         got = u_ox.sh_viewer(eye, *[torch.from_numpy(a).to(gx.DEV) for a in (pos, sh, sg, sharp, ax)], g, deg, kmax, gmax)
         np.testing.assert_allclose(got.cpu().numpy(), want, rtol=2e-5, atol=2e-6)
+
+
+def test_dist2_knn3_bit_exact(gx, orc):
+    """distCUDA2: exact three-nearest-neighbour mean, so equal to the oracle's brute force bit for
+    bit, for clustered points, duplicates, points on a plane and sizes around the box sizes."""
+    from raygaussx_amd.simple_knn import distCUDA2
+    rng = np.random.default_rng(9)
+    for n in (1, 2, 3, 4, 255, 257, 20_000):
+        _step(f"distCUDA2 n={n}")
+        p = rng.normal(size=(n, 3)).astype(np.float32)
+        if n == 20_000:
+            p[:5000] = p[:5000] * 0.01 + 3.0     # a dense cluster
+            p[5000:5100] = p[5000]               # a hundred copies of one point
+            p[6000:9000, 2] = 0.5                # a plane
+        got = distCUDA2(torch.from_numpy(p).to(gx.DEV)).cpu().numpy()
+        np.testing.assert_array_equal(got.view(np.uint32), orc.dist2_knn3(p).view(np.uint32))
+    _step("distCUDA2 n=1M")                      # full size: against a k-d tree on a sample
+    from scipy.spatial import cKDTree
+    p = scenes.scene_to_numpy(scenes.make_scene(4, n=1_000_000))["positions"]
+    got = distCUDA2(torch.from_numpy(p).to(gx.DEV)).cpu().numpy()
+    ids = rng.choice(1_000_000, 2000, replace=False)
+    d, _ = cKDTree(p.astype(np.float64)).query(p[ids].astype(np.float64), k=4)
+    np.testing.assert_allclose(got[ids], (d[:, 1:] ** 2).mean(1), rtol=1e-5)

@@ -253,3 +253,19 @@ def test_reduce_supersampling_is_the_block_mean(orc):
         np.testing.assert_allclose(got, want, rtol=0, atol=2e-7)
         if (fx, fy) == (1, 1):
             np.testing.assert_array_equal(got.reshape(-1, 3), rays)
+
+
+def test_knn3_mean_distance_matches_a_kd_tree(orc):
+    """distCUDA2 (simple_knn.cu:137-184) against scipy's cKDTree in float64 (k = 4: the point itself
+    and its three nearest), with duplicated points and fewer than four points."""
+    from scipy.spatial import cKDTree
+    rng = np.random.default_rng(3)
+    for n in (4, 50, 3000):
+        p = rng.normal(size=(n, 3)).astype(np.float32)
+        if n == 50:
+            p[10] = p[11]                       # a duplicate is a neighbour at distance 0
+        d, _ = cKDTree(p.astype(np.float64)).query(p.astype(np.float64), k=4)
+        want = (d[:, 1:] ** 2).mean(1)
+        np.testing.assert_allclose(orc.dist2_knn3(p), want, rtol=2e-6, atol=1e-12)
+    two = orc.dist2_knn3(np.array([[0, 0, 0], [1, 0, 0]], np.float32))
+    assert np.isinf(two).all()                 # (1 + FLT_MAX + FLT_MAX) / 3 overflows, as in the reference

@@ -557,12 +557,12 @@ __device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, f
     const f3 Pc = mk3(fmaf(b_inv_a, De.x, Oe.x), fmaf(b_inv_a, De.y, Oe.y), fmaf(b_inv_a, De.z, Oe.z));
     const float d2 = fmaf(Pc.x, Pc.x, fmaf(Pc.y, Pc.y, Pc.z * Pc.z));
     const float disc = 1.0f - d2;
-    if (!(disc > 1e-7f)) return false;
+    // no branch: where the line misses (disc <= 1e-7) the roots are garbage and the result false
     const float sdisc = sqrtf(disc * a);
     const float q = b + copysignf(sdisc, b);
     r1 = c / q;
     r2 = q * inv_a;
-    return true;
+    return disc > 1e-7f;
 }
 
 // A Gaussian as the shading code sees it: its record in HBM plus its rotation columns,
@@ -662,26 +662,22 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
         while (m) {
             const int c = h * 64 + __builtin_ctzll(m);
             m &= m - 1;
-            float r1, r2, t;
-            bool hit = false;
-            uint32_t in_first = 0, in_second = 0;
-            if ((Q.need && !ov) || Q.search) {
-                if (lane_roots((const float4 *)(L.tab + c * RGX_TAB), Q.dir, r1, r2)) {
-                    if (Q.search) {
-                        if (segment_hit(r1, r2, Q.slo, Q.shi, t)) found = found < 0.0f ? t : fminf(found, t);
-                    } else if (segment_hit(r1, r2, Q.tlo, Q.thi, t)) {
-                        const bool f = r1 < Q.tmid, g = r2 > Q.tmid;
-                        const bool counts = Q.part != 2 || !f;
-                        if (counts && p0 >= Q.cap) ov = true;
-                        else if (Q.part == 0 || (Q.part == 1 ? f : g)) {
-                            p0 += counts;
-                            hit = true;
-                            in_first = f ? 1u : 0u;
-                            in_second = g ? 1u : 0u;
-                        }
-                    }
-                }
-            }
+            // straight-line code: every lane evaluates both queries' predicates, its state selects
+            float r1, r2;
+            const bool ok = lane_roots((const float4 *)(L.tab + c * RGX_TAB), Q.dir, r1, r2);
+            // first-hit query (searching lanes): smallest max(slo, r1) over the entries hit in [slo, shi]
+            const float ts = fmaxf(Q.slo, r1);
+            const bool sfound = Q.search && ok && ts <= fminf(Q.shi, r2);
+            found = sfound ? (found < 0.0f ? ts : fminf(found, ts)) : found;
+            // collect query (marching lanes)
+            const bool seg = Q.need && !Q.search && !ov && ok && fmaxf(Q.tlo, r1) <= fminf(Q.thi, r2);
+            const bool f = r1 < Q.tmid, g = r2 > Q.tmid;
+            const bool counts = Q.part != 2 || !f;
+            const bool over = seg && counts && p0 >= Q.cap;
+            ov = ov || over;
+            const bool hit = seg && !over && (Q.part == 0 || (Q.part == 1 ? f : g));
+            p0 += (hit && counts) ? 1 : 0;
+            const uint32_t in_first = (hit && f) ? 1u : 0u, in_second = (hit && g) ? 1u : 0u;
             const uint64_t bal = __ballot(hit);
             if (lane == 0 && bal) cn.cands_hit++;
             if ((bal >> (row * 16)) & 0xffffull) {

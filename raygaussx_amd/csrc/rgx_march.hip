@@ -190,6 +190,8 @@ struct Frustum {
     f3 dc;       // the tile's central direction
     float delta; // no ray of the tile is further than this angle from dc
     float t0, t1, pad;
+    int32_t cut_node; // per lane: one node of the tile's cut through the tree (frustum_cut), or -1
+    int cut_n;        // nodes in the cut (wave-uniform); 0: sweeps start at the root
 };
 
 __device__ __forceinline__ f3 cross3(f3 a, f3 b) { return mk3(a.y * b.z - a.z * b.y, a.z * b.x - a.x * b.z, a.x * b.y - a.y * b.x); }
@@ -222,6 +224,8 @@ __device__ __forceinline__ void frustum_planes(const RgxCamera &cam, int px0, in
     F.o = mk3(uni(F.o.x), uni(F.o.y), uni(F.o.z));
     F.dc = mk3(uni(F.dc.x), uni(F.dc.y), uni(F.dc.z));
     F.delta = uni(F.delta);
+    F.cut_node = -1;
+    F.cut_n = 0;
 #pragma unroll
     for (int k = 0; k < 4; ++k) F.n[k] = mk3(uni(F.n[k].x), uni(F.n[k].y), uni(F.n[k].z));
 }
@@ -270,11 +274,66 @@ struct Sweep {
     int qn; // stack entries (wave-uniform)
 };
 
-__device__ __forceinline__ void sweep_begin(const MarchParams &P, Sweep &S, int32_t *s_queue)
+__device__ __forceinline__ void sweep_begin(const MarchParams &P, Sweep &S, const Frustum &F, int32_t *s_queue)
 {
-    S.qn = P.n > 0 ? 1 : 0;
-    if (threadIdx.x == 0) s_queue[0] = 0;
+    if (F.cut_n > 0) {
+        S.qn = F.cut_n;
+        if ((int)threadIdx.x < F.cut_n) s_queue[threadIdx.x] = F.cut_node;
+    } else {
+        S.qn = P.n > 0 ? 1 : 0;
+        if (threadIdx.x == 0) s_queue[0] = 0;
+    }
     __syncthreads();
+}
+
+// The tile's cut through the tree.  Every sweep of a tile tests the same top of the tree against the
+// same four planes -- a dozen steps of one to a few dozen nodes, each waiting on memory.  Done once
+// instead: descend from the root, level by level, keeping the nodes that meet the frustum at any
+// depth, until the next level would not fit one node per lane; the sweeps then start from those
+// nodes.  t_far: the largest distance any sweep of this tile will ask for (sets the planes' pad).
+__device__ __forceinline__ void frustum_cut(const MarchParams &P, Frustum &F, float t_far, int32_t *s_queue)
+{
+    const int lane = threadIdx.x;
+    const uint64_t lt = (1ull << lane) - 1ull;
+    const float4 *nodes4 = (const float4 *)P.nodes;
+    const uint32_t n_nodes = (uint32_t)(2 * P.n - 1);
+    F.t0 = 0.f;
+    F.t1 = INFINITY; // no distance shell
+    F.pad = 2.0f * RGX_PAD_REL * fmaxf(t_far, 1.0f);
+    int32_t node = lane == 0 && P.n > 0 ? 0 : -1;
+    int count = P.n > 0 ? 1 : 0;
+    for (int level = 0; level < 64 && count > 0; ++level) {
+        bool keep = false, inner = false;
+        int32_t left = 0, right = 0;
+        if ((uint32_t)node < n_nodes) {
+            const float4 a = nodes4[2 * node], b = nodes4[2 * node + 1];
+            if (frustum_overlaps(F, a, b)) {
+                left = __float_as_int(a.w);
+                inner = left >= 0;
+                keep = !inner;
+                if (inner) right = P.right[node];
+            }
+        }
+        const uint64_t bk = __ballot(keep), bi = __ballot(inner);
+        const int next = __popcll(bk) + 2 * __popcll(bi);
+        if (bi == 0 || next > 64) break; // nothing to open, or the next level does not fit: keep this one
+        // next level: the leaves kept, then the children of the inner nodes
+        if (keep) s_queue[__popcll(bk & lt)] = node;
+        if (inner) {
+            const int at = __popcll(bk) + 2 * __popcll(bi & lt);
+            s_queue[at] = left;
+            s_queue[at + 1] = right;
+        }
+        __syncthreads();
+        node = lane < next ? s_queue[lane] : -1;
+        count = next;
+        __syncthreads();
+    }
+    // nodes that failed the planes in the last round stay in the cut: the sweeps test them again
+    F.cut_n = count;
+    const uint64_t have = __ballot((uint32_t)node < n_nodes);
+    F.cut_node = node;
+    if (have != (count >= 64 ? ~0ull : ((1ull << count) - 1ull))) F.cut_n = 0; // (cannot happen) fall back to the root
 }
 
 __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int32_t *s_queue, float *s_tab, bool &done,
@@ -1004,7 +1063,7 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
             if (!split && phase == 0 && Wn.k > 1)
                 wend = fmaxf(t1, wave_max_all(want ? tlo + (float)Wn.k * R.slab_spacing : -INFINITY));
             frustum_range(F, lo, wend);
-            sweep_begin(P, S, L.queue);
+            sweep_begin(P, S, F, L.queue);
         }
         bool first = true, more = true;
         while (more) {
@@ -1028,7 +1087,7 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                     } else if (Wn.k > 1) {
                         Wn.k = 1; // too many Gaussians ahead: start over with this iteration's range only
                         frustum_range(F, t0, t1);
-                        sweep_begin(P, S, L.queue);
+                        sweep_begin(P, S, F, L.queue);
                         continue;
                     } else {
                         Wn.resident = false;
@@ -1205,6 +1264,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
     frustum_planes(P.cam, px0, py0, F);
     RayState R;
     ray_begin<false>(P, px, py, valid, R);
+    frustum_cut(P, F, wave_max_all(R.active && R.texit < 1e30f ? R.texit : 0.f), L.queue);
     const f3 dir = R.dir;
     float Cr = 0.f, Cg = 0.f, Cb = 0.f, depth = 0.f;
     Window Wn = {0.f, 0, false, 4, false};
@@ -1539,6 +1599,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
         RGX_TILE_LDS();
         Frustum F;
         frustum_planes(P.cam, px0, py0, F);
+        frustum_cut(P, F, wave_max_all(R.active && R.texit < 1e30f ? R.texit : 0.f), L.queue);
         Window Wn = {0.f, 0, false, 4, false};
         NoRecorder rec;
         while (__any(R.active)) {
@@ -1574,6 +1635,7 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
     const f3 dir = compute_ray(P.cam, (unsigned)px, (unsigned)py);
     const float tlo = valid ? seg_lo[ray] : 1.f, thi = valid ? seg_hi[ray] : 0.f;
     const bool need = valid && thi >= tlo;
+    frustum_cut(P, F, wave_max_all(need && thi < 1e30f ? thi : 0.f), L.queue);
     int p0 = 0, written = 0;
     bool ov = false;
     if (__any(need)) {

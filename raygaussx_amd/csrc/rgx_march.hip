@@ -1307,7 +1307,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
                 for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
                     const float x = sg[i] * dt;
                     const float w = __expf(-x);
-                    const float s = dt * ((1.0f - w) / fmaxf(x, 1e-6f));
+                    const float s = dt * ((1.0f - w) * __builtin_amdgcn_rcpf(fmaxf(x, 1e-6f))); // the reference's __fdividef
                     const float ts = R.T * s;
                     Cr = fmaf(ts, cr[i], Cr);
                     Cg = fmaf(ts, cg[i], Cg);
@@ -1467,7 +1467,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                     for (int i = 0; i < RGX_BUFFER_SIZE; ++i) {
                         if (i == RGX_CHUNK_SIZE) T_mid = T_after;
                         const float sd = PA[i];
-                        const float inv_d = sd > 0.0f ? 1.0f / sd : 0.0f;
+                        const float inv_d = sd > 0.0f ? __builtin_amdgcn_rcpf(sd) : 0.0f;
                         const float e = PB[i] * inv_d;
                         const float w = __expf(-sd * dt);
                         const float a = T_after * (1.0f - w) * inv_d;
@@ -1496,7 +1496,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                     const f3 inv_s = mk3(inv.x * k, inv.y * k, inv.z * k);
                     const float cut = k * k;
                     const float rho = col.w;
-                    const float dcg = dot3(mk3(col.x, col.y, col.z), g) / rho;
+                    const float dcg = dot3(mk3(col.x, col.y, col.z), g) * __builtin_amdgcn_rcpf(rho);
                     // mask recurrence exactly as backward/gaussians_aabb.cu:375-396, 437-438
                     const f3 Us = U * inv_s.x, Vs = V * inv_s.y, Ws = W * inv_s.z;
                     const f3 M1 = mk3(Us.x, Vs.x, Ws.x), M2 = mk3(Us.y, Vs.y, Ws.y), M3 = mk3(Us.z, Vs.z, Ws.z);

@@ -372,8 +372,9 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
             quat_to_cols(p.quat4, U, V, W);
             const f3 O = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
             // semi-axes of the k-sigma ellipsoid: k * scale = 1 / inv_inter
-            const f3 ax = mk3(1.0f / p.inv_inter4.x, 1.0f / p.inv_inter4.y, 1.0f / p.inv_inter4.z);
-            const float dist = sqrtf(dot3(O, O));
+            // (bounds only: hardware reciprocal and square root, their last-bit error is inside the 1.001 factors)
+            const f3 ax = mk3(__builtin_amdgcn_rcpf(p.inv_inter4.x), __builtin_amdgcn_rcpf(p.inv_inter4.y), __builtin_amdgcn_rcpf(p.inv_inter4.z));
+            const float dist = __builtin_amdgcn_sqrtf(dot3(O, O));
             const float amax = fmaxf(ax.x, fmaxf(ax.y, ax.z));
             const float rad = amax * 1.001f + 1e-5f * dist + F.pad;
             // Along a ray of direction d the ellipsoid lies within (centre - eye).d -+ |A R^T d|.  For
@@ -383,8 +384,8 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
             const float depth = -dot3(O, F.dc);
             const f3 off = mk3(-O.x - depth * F.dc.x, -O.y - depth * F.dc.y, -O.z - depth * F.dc.z);
             const float eu = dot3(U, F.dc) * ax.x, ev = dot3(V, F.dc) * ax.y, ew = dot3(W, F.dc) * ax.z;
-            const float ext = sqrtf((eu * eu + ev * ev) + ew * ew) * 1.001f;
-            const float slack = 1.5f * (0.5f * fabsf(depth) * F.delta * F.delta + (sqrtf(dot3(off, off)) + amax) * F.delta) +
+            const float ext = __builtin_amdgcn_sqrtf((eu * eu + ev * ev) + ew * ew) * 1.001f;
+            const float slack = 1.5f * (0.5f * fabsf(depth) * F.delta * F.delta + (__builtin_amdgcn_sqrtf(dot3(off, off)) + amax) * F.delta) +
                                 1e-5f * dist + F.pad;
             dmin = fmaxf(dist - rad, depth - ext - slack);
             dmax = fminf(dist + rad, depth + ext + slack);
@@ -395,7 +396,7 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
                 const f3 n = F.n[k];
                 // the ellipsoid reaches h beyond its centre along n; centre - eye = -O
                 const float hu = dot3(U, n) * ax.x, hv = dot3(V, n) * ax.y, hw = dot3(W, n) * ax.z;
-                const float h = sqrtf((hu * hu + hv * hv) + hw * hw) * 1.001f;
+                const float h = __builtin_amdgcn_sqrtf((hu * hu + hv * hv) + hw * hw) * 1.001f;
                 ok = ok && !(-dot3(n, O) - h > F.pad);
             }
             leaf_hit = ok;

@@ -1,22 +1,25 @@
-// Ray-march kernels: forward compositing and the replaying backward pass.
+// Ray-march kernels: forward compositing, its viewer variant, and the two backward passes.
 // Replace the OptiX programs of optix_raycasting/cuda_train/forward/gaussians_aabb.cu
-// (also cuda_test/, byte-identical) and cuda_train/backward/gaussians_aabb.cu, and
-// their launchers (optix_raycasting/optix_utils.py:222-322, 363-500, 503-601).
+// (also cuda_test/, byte-identical), cuda_gui/gaussians_aabb.cu and
+// cuda_train/backward/gaussians_aabb.cu, and their launchers
+// (optix_raycasting/optix_utils.py:222-322, 363-500, 503-601).
 //
 // Mapping: one lane per ray, one 64-lane wavefront (= one workgroup) per 8x8 pixel
 // tile, all rays of a tile sharing the camera origin.  Per slab iteration the wave
-//   1. gathers, cooperatively, the Gaussians whose boxes meet the tile's frustum
-//      over the union of the lanes' slab intervals: a 64-wide sweep of the BVH with
-//      the node stack and the candidate table in LDS (one node per lane per step);
-//   2. walks the candidate table in lock step: every lane evaluates the exact hit
-//      predicate for ITS ray and slab (so hit sets are those of a per-ray query),
-//      and the lanes that hit accumulate the candidate's samples.  Candidate data
-//      is wave-uniform, i.e. one 64-byte fetch per wave instead of one per lane;
-//   3. (backward) sums each candidate's 14 gradient words over the 16 rays of a 4x4
-//      pixel row with DPP adds and issues ONE set of atomics per row and candidate.
-// The first-hit query (once per ray, and after an empty slab) runs on the same
-// candidate tables.  The per-lane skip-link queries below serve the segment test
-// hooks (arbitrary rays).
+//   1. makes its candidate table (LDS) cover the lanes' slab intervals: it reuses the resident
+//      window, or sweeps the BVH cooperatively (node stack in LDS, one node per lane per step,
+//      starting from the tile's cut through the tree) for the Gaussians whose ellipsoids meet
+//      the tile's frustum in the depth range wanted;
+//   2. filters: a wave-uniform loop over the table in which every lane evaluates the exact hit
+//      predicate for ITS ray and slab (so hit sets are those of a per-ray query); the result is,
+//      per 4x4 pixel row, the list of entries hit, and per lane its hit bits over that list;
+//   3. shades: every lane walks its own hits (forward, the backward's density pass), or the four
+//      rows walk their lists in lock step and sum each entry's 14 gradient words over the row's
+//      16 rays with DPP adds (the backward's gradient pass).
+// The forward can record what 1 and 2 produced; the replaying backward then needs no tree, no
+// table and no predicate, and sums a window's gradients in LDS before adding them to memory.
+// The first-hit query (once per ray, and after an empty slab) runs on the same candidate tables.
+// The per-lane skip-link queries below serve the segment test hooks (arbitrary rays).
 #include "rgx_device.h"
 
 #include <type_traits>

@@ -140,7 +140,8 @@ int rgx_march_workspace_bytes(int64_t n, int64_t n_rays, int32_t max_prim_slice,
  * 32-bit words (>= 1024, multiple of 4; 16384 is ample for the benchmark scenes) holding, per
  * slab iteration, which Gaussians each 4x4 pixel row hits and each ray's hit bits.  A backward
  * given the record of its forward replays those lists instead of searching the tree again;
- * tiles whose region overflowed are recomputed.  The role the reference's hit_prim_idx buffer
+ * tiles whose region overflowed, or whose region was not written by a forward launch with the same
+ * number of Gaussians, image size and step, are recomputed.  The role the reference's hit_prim_idx buffer
  * plays between its collect and blend steps (optix_utils.py:306), at a few hundred bytes per
  * tile and slab instead of max_prim_slice ints per ray. */
 int rgx_march_records_bytes(int32_t width, int32_t height, int32_t tile_words, size_t *bytes);

@@ -839,6 +839,20 @@ __device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds 
 #define RGX_REC_LISTS 0x4C000000u
 #define RGX_REC_TRAIL 0x54000000u
 
+// Words 2 and 3 of a tile's region name the launch the record belongs to (number of Gaussians,
+// image size, step), so that a backward handed a record of another scene or view recomputes the
+// tile instead of following indices that mean nothing in its own tables.
+__device__ __forceinline__ uint32_t record_mark(const MarchParams &P, int which)
+{
+    return which == 0 ? (uint32_t)P.n : ((uint32_t)P.cam.width << 16 ^ (uint32_t)P.cam.height ^ __float_as_uint(P.m.dt_step));
+}
+__device__ __forceinline__ bool record_usable(const MarchParams &P, const uint32_t *reg)
+{
+    return (uint32_t)__builtin_amdgcn_readfirstlane((int)reg[0]) == 0u &&
+           (uint32_t)__builtin_amdgcn_readfirstlane((int)reg[2]) == record_mark(P, 0) &&
+           (uint32_t)__builtin_amdgcn_readfirstlane((int)reg[3]) == record_mark(P, 1);
+}
+
 struct Recorder {
     uint32_t *reg;  // this tile's region, or null
     int off;        // next free word (wave-uniform)
@@ -898,11 +912,13 @@ struct Recorder {
         off += 4 + (any_search ? 64 : 0);
     }
 
-    __device__ __forceinline__ void finish()
+    __device__ __forceinline__ void finish(const MarchParams &P)
     {
         if (reg && threadIdx.x == 0) {
             reg[0] = ovf ? 1u : 0u;
             reg[1] = (uint32_t)off;
+            reg[2] = record_mark(P, 0);
+            reg[3] = record_mark(P, 1);
         }
     }
 };
@@ -912,7 +928,7 @@ struct NoRecorder {
     __device__ __forceinline__ void write_window(const TileLds &, int) {}
     __device__ __forceinline__ void write_lists(const TileLds &, int, bool) {}
     __device__ __forceinline__ void write_trailer(bool, float, float) {}
-    __device__ __forceinline__ void finish() {}
+    __device__ __forceinline__ void finish(const MarchParams &) {}
 };
 
 __device__ __forceinline__ uint32_t uni_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
@@ -950,7 +966,7 @@ __device__ __forceinline__ void replay_window(const MarchParams &P, const Replay
     if (at == win_at) return;
     replay_flush(P, RL);
     const int C = (int)(uni_u32(reg[at]) & 0xffffu);
-    for (int i = threadIdx.x; i < C && i < RGX_CCAP; i += 64) RL.pid[i] = reg[at + 4 + i];
+    for (int i = threadIdx.x; i < C && i < RGX_CCAP; i += 64) RL.pid[i] = min(reg[at + 4 + i], (uint32_t)(P.n - 1));
     win_at = at;
     __syncthreads();
 }
@@ -970,7 +986,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
     const uint8_t *slots = (const uint8_t *)(it + 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0));
     const uint32_t *masks = it + 8 + q0 + q1 + q2 + q3 + lane; // word w of this lane: masks[w * 64]
     if constexpr (WALK != WALK_ROWS_ALL) {
-        const int nwr = run ? (len + 31) >> 5 : 0; // words of this lane's row; later words are not its own
+        const int nwr = run ? min((len + 31) >> 5, nw) : 0; // words of this lane's row; later words are not its own
         const uint32_t *half = it + 8 + q0 + q1 + q2 + q3 + nw * 64 + ((WALK & 1) * 4 + row) * nw;
         auto word = [&](int w) { return WALK == WALK_LANES_ALL ? masks[w * 64] : masks[w * 64] & half[w]; };
         if (COUNT)
@@ -983,14 +999,14 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
             if (!__any(has)) break;
             int slot = 0;
             if (has) {
-                slot = slots[w * 32 + __builtin_ctz(bits)];
+                slot = slots[w * 32 + __builtin_ctz(bits)] & (RGX_CCAP - 1);
                 bits &= bits - 1u;
             }
             const int32_t pid = (int32_t)RL.pid[slot];
             body(Entry<false>{nullptr, P.prims + pid, pid, slot}, has, has, Half<(WALK & 1)>{});
         }
     } else {
-        const int maxlen = max(max(l0, l1), max(l2, l3));
+        const int maxlen = min(max(max(l0, l1), max(l2, l3)), nw * 32);
         uint32_t bits = 0;
         for (int i = 0; i < maxlen; ++i) {
             if ((i & 31) == 0) bits = masks[(i >> 5) * 64];
@@ -998,7 +1014,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
             const bool hit = run && live && ((bits >> (i & 31)) & 1u);
             if (COUNT && hit) ++p0;
             if (__ballot(hit)) {
-                const int slot = live ? slots[i] : 0;
+                const int slot = live ? slots[i] & (RGX_CCAP - 1) : 0;
                 const int32_t pid = (int32_t)RL.pid[slot];
                 body(Entry<false>{nullptr, P.prims + pid, pid, slot}, hit, live, Half<0>{});
             }
@@ -1355,7 +1371,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
             P.ray_colors[3 * ray + 2] = Cb + R.T * bg;
         }
     }
-    rec.finish();
+    rec.finish(P);
     flush_stats(P.stats, cn);
 }
 
@@ -1394,9 +1410,9 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
     if (!tile_origin(P, px0, py0, &tile)) return; // whole wave
     const uint32_t *reg = P.records ? P.records + (int64_t)tile * P.rec_tile_words : nullptr;
     if (REPLAY) {
-        if (uni_u32(reg[0]) != 0u) return; // this tile's record overflowed: the other kernel handles it
+        if (!record_usable(P, reg)) return; // overflowed, or not this launch's: the other kernel handles the tile
     } else if (P.only_overflow) {
-        if (uni_u32(reg[0]) == 0u) return; // replayed
+        if (record_usable(P, reg)) return; // replayed
     }
     const int lane = threadIdx.x;
     __shared__ float s_acc[REPLAY ? 14 * RGX_CCAP : 1];
@@ -1404,6 +1420,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
     const ReplayLds RL = {s_acc, s_pid, s_touched};
     if constexpr (REPLAY) {
         for (int i = lane; i < 14 * RGX_CCAP; i += 64) s_acc[i] = 0.f;
+        for (int i = lane; i < RGX_CCAP; i += 64) s_pid[i] = 0u;
         if (lane < RGX_CCAP / 32) s_touched[lane] = 0u;
         __syncthreads();
     }

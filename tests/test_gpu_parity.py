@@ -311,6 +311,41 @@ def test_backward_replay_of_recorded_hit_lists_equals_recomputation(gx, orc):
             assert cos >= 1 - 1e-9 and rel <= 2e-5, (label, k, cos, rel)
 
 
+def test_backward_ignores_a_record_of_another_launch(gx):
+    """A record names the launch it belongs to; handed the record of another scene (or step), the
+    backward searches the tree for every tile, as without a record, instead of replaying it."""
+    from raygaussx_amd import optix_utils as u_ox
+    from raygaussx_amd.render_optix import compute_rgb
+    cam = scenes.make_camera(0, 0, width=40, height=32)
+    cs = u_ox.camera_struct(cam)
+    dloss = torch.from_numpy(np.random.default_rng(1).normal(size=(40 * 32, 3)).astype(np.float32)).to(gx.DEV)
+
+    def launch(n, seed, dt, records_from=None):
+        sc = gx.to_dev(scenes.scene_to_numpy(scenes.make_scene(0, n=n, sh_degree=0, seed=seed)))
+        gas = u_ox.AccelerationStructure(n, gx.DEV).build_from_gaussians(sc["positions"], sc["scales"] * 1.5,
+                                                                          sc["quaternions"], sc["densities"])
+        rgb = compute_rgb(cam.camera_center, sc["positions"], sc["color_features"], None, None, None, 0, 0)
+        ps = u_ox.pack_prims(gas, cs, sc["positions"], sc["scales"] * 1.5, sc["quaternions"], sc["densities"], rgb)
+        rec = u_ox.new_records(cs, gx.DEV)
+        img = u_ox.march_forward(gas, cs, ps, dt, False, 512, True, records=rec)
+        stats = u_ox.new_stats(gx.DEV)
+        grads = u_ox.march_backward(gas, cs, ps, img, dloss, dt, False, 512, True, stats=stats,
+                                    records=rec if records_from is None else records_from)
+        return rec, [g.cpu().numpy() for g in grads], u_ox.read_stats(stats)
+
+    _step("backward with its own record")
+    rec_a, own, st_own = launch(3000, 5, 0.004)
+    assert st_own["nodes_visited"] == 0 and st_own["hit_pairs"] > 10000
+    for label, n, seed, dt in (("another scene", 2500, 6, 0.004), ("another step", 3000, 5, 0.005)):
+        _step("backward with the record of " + label)
+        _, ref, st_ref = launch(n, seed, dt)                       # its own record: the expected gradients
+        _, got, st = launch(n, seed, dt, records_from=rec_a)       # the foreign one
+        assert st["nodes_visited"] > 0 and st["replay_lost"] == 0 and st["hit_pairs"] == st_ref["hit_pairs"]
+        for g, r in zip(got, ref):
+            cos, rel = gx.cos_rel(g, r)
+            assert cos >= 1 - 1e-6 and rel <= 1e-4
+
+
 def test_dynamic_sampling_lobes_supersampling_black_background(gx, orc):
     """The unbounded-scene settings (adaptive step, camera inside the cloud) with spherical-Gaussian
     lobes, a non-multiple-of-8 image, 2x1 supersampling and a black background."""

@@ -572,3 +572,52 @@ def test_dist2_knn3_bit_exact(gx, orc):
     ids = rng.choice(1_000_000, 2000, replace=False)
     d, _ = cKDTree(p.astype(np.float64)).query(p[ids].astype(np.float64), k=4)
     np.testing.assert_allclose(got[ids], (d[:, 1:] ** 2).mean(1), rtol=1e-5)
+
+
+def test_training_loop_as_the_reference_writes_it_reduces_the_loss(gx):
+    """scripts/train.py:101-148 in miniature: OptiX set-up calls, RenderOptixSettings with the
+    reference's positional arguments, RenderOptixFunction.apply on activated parameters, an L1 loss,
+    Adam.  A perturbed copy of a scene must move back towards the images of the original."""
+    from raygaussx_amd import optix_utils as u_ox
+    from raygaussx_amd.render_optix import RenderOptixFunction, RenderOptixSettings
+    torch.manual_seed(0)
+    truth = {k: v.to(gx.DEV) for k, v in scenes.make_scene(0, n=1500, sh_degree=1, seed=31).items()}
+    truth["scales"] = truth["scales"] * 2.0
+    cams = [scenes.make_camera(1, i, width=48, height=48).to(gx.DEV) for i in (0, 17, 43, 71)]
+    ctx = u_ox.create_context(log=None)
+    mod_f, mod_b = u_ox.create_module(ctx, None, stage="forward"), u_ox.create_module(ctx, None, stage="backward")
+    pg_f, pg_b = u_ox.create_program_groups(ctx, mod_f), u_ox.create_program_groups(ctx, mod_b)
+    pl_f, pl_b = u_ox.create_pipeline(ctx, pg_f, None), u_ox.create_pipeline(ctx, pg_b, None)
+    empty = (torch.zeros(1500, 3, 0, device=gx.DEV), torch.zeros(1500, 0, device=gx.DEV), torch.zeros(1500, 0, 3, device=gx.DEV))
+
+    def render(p, cam):
+        settings = RenderOptixSettings(ctx, False, None, pg_f, pl_f, pg_b, pl_b, 0.005, False, cam, 512, 0, 0, 0, 0,
+                                       (1, 1), True, None)
+        quat = torch.nn.functional.normalize(p["quaternions"], dim=1)
+        return RenderOptixFunction.apply(p["positions"], torch.exp(p["log_scales"]), quat, p["densities"],
+                                         p["color_features"], *empty, settings)
+
+    with torch.no_grad():
+        t = dict(truth, log_scales=truth["scales"].log())
+        targets = [render(t, c) for c in cams]
+    params = {"positions": truth["positions"] + 0.01 * torch.randn_like(truth["positions"]),
+              "log_scales": truth["scales"].log() + 0.1 * torch.randn_like(truth["scales"]),
+              "quaternions": truth["quaternions"] + 0.05 * torch.randn_like(truth["quaternions"]),
+              "densities": truth["densities"] * (1 + 0.2 * torch.randn_like(truth["densities"])).clamp(min=0.3),
+              "color_features": truth["color_features"] + 0.1 * torch.randn_like(truth["color_features"])}
+    params = {k: v.clone().requires_grad_(True) for k, v in params.items()}
+    opt = torch.optim.Adam([{"params": [params["positions"]], "lr": 2e-4}, {"params": [params["log_scales"]], "lr": 5e-3},
+                            {"params": [params["quaternions"]], "lr": 2e-3}, {"params": [params["densities"]], "lr": 1e-2},
+                            {"params": [params["color_features"]], "lr": 5e-3}])
+    _step("60 Adam steps")
+    losses = []
+    for it in range(60):
+        cam, target = cams[it % 4], targets[it % 4]
+        loss = (render(params, cam) - target).abs().mean()
+        opt.zero_grad()
+        loss.backward()
+        opt.step()
+        losses.append(loss.item())
+        assert all(torch.isfinite(p.grad).all() for p in params.values())
+    first, last = np.mean(losses[:4]), np.mean(losses[-4:])
+    assert last < 0.6 * first, (first, last)

@@ -40,7 +40,7 @@ HBM_PEAK_GBPS = 8000.0
 # profiles/march_kernels_c4_1M_800x800.md.  Workloads without a measurement report null.
 MEASURED_TRAFFIC_BYTES = {
     ("c4_1M_800x800", "march_backward"): 11.8e9,   # k_march_bwd_replay: 3.2 GB read, 8.6 GB written
-    ("c4_1M_800x800", "march_forward"): 3.39e9,    # k_march_fwd<true, false>: 2.0 GB read, 1.4 GB written (0.9 the record)
+    ("c4_1M_800x800", "march_forward"): 3.39e9,    # k_march_fwd<true, false>: 2.0 GB read, 1.4 GB written (0.23 the record)
 }
 
 WORKLOADS = {

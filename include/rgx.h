@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define RGX_ABI_VERSION 2
+#define RGX_ABI_VERSION 3
 
 #define RGX_OK 0
 #define RGX_EINVAL -1     /* bad argument (null pointer, negative size, unsupported degree ...) */

@@ -791,22 +791,17 @@ __device__ __forceinline__ void shade_rows(const MarchParams &P, const TileLds &
 // For bodies that need no sum over the rays of a row.  The order of a ray's hits is that of
 // shade_rows.  Only the entries that can reach half `half` of the slab's samples are visited; the
 // body gets Half<TAG>.
-#ifdef RGX_NOHALF_WALK
-#define RGX_HALF(x) 0xffffffffu
-#else
-#define RGX_HALF(x) (x)
-#endif
 template <int TAG, typename Body>
 __device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds &L, int len, bool run, int half, Body body)
 {
     const int lane = threadIdx.x, row = lane >> 4;
     const int nw = (len + 31) >> 5;
     int w = 0;
-    uint32_t bits = (run && nw > 0) ? L.mask[0][lane] & RGX_HALF(L.half[half][row][0]) : 0u;
+    uint32_t bits = (run && nw > 0) ? L.mask[0][lane] & L.half[half][row][0] : 0u;
     for (;;) {
         while (bits == 0u && run && w + 1 < nw) {
             ++w;
-            bits = L.mask[w][lane] & RGX_HALF(L.half[half][row][w]);
+            bits = L.mask[w][lane] & L.half[half][row][w];
         }
         const bool has = bits != 0u;
         if (!__any(has)) break;

@@ -75,6 +75,60 @@ def cpu_baseline(scene, cam, cfg, n_sample, threads, backward=True):
                        f"(brute-force hit search), {dt:.1f} s")
 
 
+def _timed(fn, reps):
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps * 1e3
+
+
+def side_kernels(dev, reps):
+    """The entry points either side of the march, each on its benchmark-size input: ms per call and, for
+    the streaming ones, algorithmic bytes moved per second against the 8 TB/s of HBM."""
+    from raygaussx_amd.general_utils import reduce_supersampling
+    from raygaussx_amd.reordering import morton_order, reorder_tensors
+    from raygaussx_amd.render_optix import compute_rgb
+    from raygaussx_amd.simple_knn import distCUDA2
+    out = {}
+    # image epilogue: 1920x1080 at 2x2 supersampling -> float image + 8-bit image
+    w, h, f = 1920, 1080, (2, 2)
+    rays = torch.rand(w * f[0] * h * f[1], 3, device=dev)
+    ms = _timed(lambda: reduce_supersampling(w, h, rays, f, clip=True, to_uint8=True), reps)
+    nbytes = rays.numel() * 4 + w * h * 3 * 5
+    out["reduce_supersampling_1080p_2x2"] = dict(ms=round(ms, 4), GBps=round(nbytes / ms / 1e6, 1), frac_hbm=round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4))
+    # reordering of a 1 M point cloud: parameters + two Adam moments each (classes/point_cloud.py:1031-1044)
+    sc = {k: v.to(dev) for k, v in scenes.make_scene(4, n=1_000_000).items()}
+    tensors = [sc[k] for k in ("positions", "scales", "quaternions", "densities", "color_features")]
+    tensors = tensors + [t.clone() for t in tensors] + [t.clone() for t in tensors]
+    out["morton_order_1M"] = dict(ms=round(_timed(lambda: morton_order(sc["positions"]), reps), 4))
+    order = morton_order(sc["positions"])
+    ms = _timed(lambda: reorder_tensors(order, tensors), reps)
+    nbytes = 2 * sum(t.numel() * 4 for t in tensors) + order.numel() * 8
+    out["reorder_tensors_1M_x15"] = dict(ms=round(ms, 4), GBps=round(nbytes / ms / 1e6, 1), frac_hbm=round(nbytes / ms / 1e6 / HBM_PEAK_GBPS, 4))
+    ms_torch = _timed(lambda: [t.index_select(0, order) for t in tensors], reps)
+    out["reorder_tensors_1M_x15"]["torch_index_select_ms"] = round(ms_torch, 4)
+    # distCUDA2 at 1 M and 3 M points
+    out["distCUDA2_1M"] = dict(ms=round(_timed(lambda: distCUDA2(sc["positions"]), reps), 4))
+    big = scenes.make_scene(3)
+    pos3 = big["positions"].to(dev)
+    out["distCUDA2_3M"] = dict(ms=round(_timed(lambda: distCUDA2(pos3), reps), 4))
+    # viewer launch on the 3 M scene at 1920x1080 (tree built once)
+    cfg = scenes.CONFIGS[3]
+    d3 = {k: v.to(dev) for k, v in big.items()}
+    tree = u_ox.AccelerationStructure(d3["positions"].shape[0], dev).build_from_gaussians(d3["positions"], d3["scales"],
+                                                                                            d3["quaternions"], d3["densities"])
+    cam = scenes.make_camera(3, 0).to(dev)
+    cs = u_ox.camera_struct(cam)
+    rgb = compute_rgb(cam.camera_center, d3["positions"], d3["color_features"], None, None, None, 0, 3)
+    prims = u_ox.pack_prims(tree, cs, d3["positions"], d3["scales"], d3["quaternions"], d3["densities"], rgb)
+    ms = _timed(lambda: u_ox.march_viewer(tree, cs, prims, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"], cfg["t_eps"]), reps)
+    out["march_viewer_c3_1080p"] = dict(ms=round(ms, 4), frames_per_s=round(1e3 / ms, 2))
+    return dict(side_kernels=out, reps=reps, data="synthetic")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -85,6 +139,9 @@ def main():
     ap.add_argument("--forward-only", action="store_true")
     ap.add_argument("--no-records", action="store_true",
                     help="backward searches the tree again instead of replaying the forward's hit-list record")
+    ap.add_argument("--side-kernels", action="store_true",
+                    help="time the entry points around the march (image epilogue, reorder gather, distCUDA2, viewer launch) "
+                         "instead of the training step; one JSON line")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a 1 GiB device-to-device copy (reference reading for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -103,6 +160,9 @@ def main():
         print(json.dumps(dict(calibration="copy", bytes_read=src.numel() * 4, bytes_written=dst.numel() * 4, launches=3)))
         return
     L.lib()
+    if args.side_kernels:
+        print(json.dumps(side_kernels(dev, args.steps)), flush=True)
+        return
     config, n, width, height = WORKLOADS[args.workload]
     cfg = dict(scenes.CONFIGS[config])
     scene = scenes.make_scene(config, n=n)

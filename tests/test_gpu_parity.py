@@ -621,3 +621,70 @@ def test_training_loop_as_the_reference_writes_it_reduces_the_loss(gx):
         assert all(torch.isfinite(p.grad).all() for p in params.values())
     first, last = np.mean(losses[:4]), np.mean(losses[-4:])
     assert last < 0.6 * first, (first, last)
+
+
+def test_direct_ctypes_binding_matches_the_python_mirror(gx, c0):
+    """The stand-alone ctypes stub a maintainer would write (no raygaussx_amd imports in the call
+    path): build, colour, pack, forward with a record, backward, colour gradient -- equal to what
+    RenderOptixFunction returns for the same inputs."""
+    import ctypes as C
+    from raygaussx_amd import _lib
+    lib = C.CDLL(_lib.LIB_PATH)
+
+    class RgxCamera(C.Structure):
+        _fields_ = [("eye", C.c_float * 3), ("u", C.c_float * 3), ("v", C.c_float * 3), ("w", C.c_float * 3),
+                    ("tan_half_fov_x", C.c_float), ("tan_half_fov_y", C.c_float),
+                    ("principal_x", C.c_float), ("principal_y", C.c_float),
+                    ("width", C.c_int32), ("height", C.c_int32)]
+
+    class RgxMarch(C.Structure):
+        _fields_ = [("dt_step", C.c_float), ("dynamic_sampling", C.c_int32), ("max_prim_slice", C.c_int32),
+                    ("white_background", C.c_int32), ("t_eps", C.c_float)]
+
+    def p(t):
+        return C.c_void_p(t.data_ptr())
+
+    def ws(fn, *a):
+        n = C.c_size_t()
+        assert fn(*a, C.byref(n)) == 0
+        return torch.empty(n.value, dtype=torch.uint8, device=gx.DEV)
+
+    sc, camera, cfg = c0
+    d = gx.to_dev(sc)
+    pos, scale, quat, dens, sh = (d[k] for k in ("positions", "scales", "quaternions", "densities", "color_features"))
+    N, W, H = pos.shape[0], camera.image_width, camera.image_height
+    rot = camera.world_view_transform[:3, :3]
+    import math
+    cam = RgxCamera((C.c_float * 3)(*camera.camera_center.tolist()), (C.c_float * 3)(*rot[:, 0].tolist()),
+                    (C.c_float * 3)(*rot[:, 1].tolist()), (C.c_float * 3)(*rot[:, 2].tolist()),
+                    math.tan(camera.FoVx / 2), math.tan(camera.FoVy / 2), camera.Px, camera.Py, W, H)
+    march = RgxMarch(cfg["dt_step"], 0, cfg["max_prim_slice"], 1, 1e-3)
+    s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    bvh = ws(lib.rgx_build_workspace_bytes, C.c_int64(N))
+    mws = ws(lib.rgx_march_workspace_bytes, C.c_int64(N), C.c_int64(W * H), C.c_int32(cfg["max_prim_slice"]))
+    rec = ws(lib.rgx_march_records_bytes, C.c_int32(W), C.c_int32(H), C.c_int32(16384))
+    eye = (C.c_float * 3)(*camera.camera_center.tolist())
+    f = dict(dtype=torch.float32, device=gx.DEV)
+    rgb, prims, img = torch.empty(N, 3, **f), torch.empty(N, 16, **f), torch.empty(W * H, 3, **f)
+    dimg = torch.from_numpy(np.random.default_rng(2).normal(size=(W * H, 3)).astype(np.float32)).to(gx.DEV)
+    ddens, drgb, dpos, dscale, dquat = (torch.empty(N, **f), torch.empty(N, 3, **f), torch.empty(N, 3, **f),
+                                        torch.empty(N, 3, **f), torch.empty(N, 4, **f))
+    dsh, dpos_dir = torch.empty_like(sh), torch.empty(N, 3, **f)
+    _step("direct ctypes calls")
+    assert lib.rgx_build(p(pos), p(scale), p(quat), p(dens), C.c_int64(N), C.c_float(0.1), p(bvh), C.c_size_t(bvh.numel()), s) == 0
+    assert lib.rgx_sh_forward(eye, p(pos), p(sh), None, None, None, 0, 3, C.c_int64(N), p(rgb), s) == 0
+    assert lib.rgx_pack_prims(p(bvh), eye, p(pos), p(scale), p(quat), p(dens), p(rgb), C.c_int64(N), C.c_float(0.1), p(prims), s) == 0
+    assert lib.rgx_march_forward(p(bvh), C.byref(cam), C.byref(march), p(prims), C.c_int64(N), p(img),
+                                 p(mws), C.c_size_t(mws.numel()), p(rec), C.c_size_t(rec.numel()), None, s) == 0
+    assert lib.rgx_march_backward(p(bvh), C.byref(cam), C.byref(march), p(prims), C.c_int64(N), p(img), p(dimg),
+                                  p(ddens), p(drgb), p(dpos), p(dscale), p(dquat), p(mws), C.c_size_t(mws.numel()),
+                                  p(rec), C.c_size_t(rec.numel()), None, s) == 0
+    assert lib.rgx_sh_backward(eye, p(pos), p(sh), None, None, None, 0, 3, C.c_int64(N), p(drgb),
+                               p(dsh), p(dpos_dir), None, None, None, s) == 0
+    dpos += dpos_dir
+    torch.cuda.synchronize()
+    ref = gx.gpu_render(sc, camera, cfg, want_grad=dimg.cpu().numpy(), stats=False)
+    np.testing.assert_array_equal(img.cpu().numpy(), ref["image"])
+    for name, got in (("positions", dpos), ("scales", dscale), ("quaternions", dquat), ("densities", ddens), ("color_features", dsh)):
+        cos, rel = gx.cos_rel(got.cpu().numpy(), ref["grads"][name])
+        assert cos >= 1 - 1e-6 and rel <= 1e-4, (name, cos, rel)

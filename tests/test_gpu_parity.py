@@ -688,3 +688,23 @@ def test_direct_ctypes_binding_matches_the_python_mirror(gx, c0):
     for name, got in (("positions", dpos), ("scales", dscale), ("quaternions", dquat), ("densities", ddens), ("color_features", dsh)):
         cos, rel = gx.cos_rel(got.cpu().numpy(), ref["grads"][name])
         assert cos >= 1 - 1e-6 and rel <= 1e-4, (name, cos, rel)
+
+
+def test_empty_cloud_and_one_pixel_image(gx):
+    """No Gaussians at all renders the background and returns empty gradients; a 1x1 image works."""
+    cam = scenes.make_camera(0, 0, width=16, height=8)
+    cfg = dict(dt_step=0.0025, dynamic_sampling=False, max_prim_slice=64)
+    empty = {k: v[:0].copy() for k, v in scenes.scene_to_numpy(scenes.make_scene(0, n=4, sh_degree=1, seed=1)).items()
+             if k in ("positions", "scales", "quaternions", "densities", "color_features")}
+    _step("empty cloud")
+    out = gx.gpu_render(empty, cam, cfg, want_grad=np.ones((16 * 8, 3), np.float32))
+    np.testing.assert_array_equal(out["image"], 1.0)
+    assert out["grads"]["positions"].shape == (0, 3) and out["grads"]["color_features"].shape == (0, 3, 4)
+    _step("1x1 image")
+    sc = scenes.scene_to_numpy(scenes.make_scene(0, n=300, sh_degree=0, seed=2))
+    sc["scales"] = sc["scales"] * 3
+    cam1 = scenes.make_camera(0, 0, width=1, height=1)
+    out = gx.gpu_render(sc, cam1, cfg, want_grad=np.ones((1, 3), np.float32))
+    assert out["image"].shape == (1, 3) and np.isfinite(out["image"]).all()
+    assert out["stats_fwd"]["hit_pairs"] == out["stats_bwd"]["hit_pairs"] > 0
+    assert np.isfinite(out["grads"]["positions"]).all() and np.abs(out["grads"]["positions"]).sum() > 0

@@ -274,11 +274,13 @@ __device__ __forceinline__ bool frustum_overlaps(const Frustum &F, float4 a, flo
 // when the stack is empty (done) or the table might not take another step's leaves; call again
 // to continue with an emptied table.
 struct Sweep {
-    int qn; // stack entries (wave-uniform)
+    int qn;  // stack entries (wave-uniform)
+    int lqn; // leaves waiting for their ellipsoid test (wave-uniform)
 };
 
 __device__ __forceinline__ void sweep_begin(const MarchParams &P, Sweep &S, const Frustum &F, int32_t *s_queue)
 {
+    S.lqn = 0;
     if (F.cut_n > 0) {
         S.qn = F.cut_n;
         if ((int)threadIdx.x < F.cut_n) s_queue[threadIdx.x] = F.cut_node;
@@ -339,15 +341,77 @@ __device__ __forceinline__ void frustum_cut(const MarchParams &P, Frustum &F, fl
     if (have != (count >= 64 ? ~0ull : ((1ull << count) - 1ull))) F.cut_n = 0; // (cannot happen) fall back to the root
 }
 
-__device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int32_t *s_queue, float *s_tab, bool &done,
-                          Counters &cn)
+__device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int32_t *s_queue, int32_t *s_leafq, float *s_tab,
+                          bool &done, Counters &cn)
 {
     const int lane = threadIdx.x;
     const uint64_t lt = (1ull << lane) - 1ull;
     const float4 *nodes4 = (const float4 *)P.nodes;
     const uint32_t n_nodes = (uint32_t)(2 * P.n - 1);
     int C = 0;
-    while (S.qn > 0 && C + 64 <= RGX_CCAP) {
+    while ((S.qn > 0 || S.lqn > 0) && C + 64 <= RGX_CCAP) {
+        if (S.lqn >= 64 || S.qn == 0) {
+            // Leaves whose boxes passed wait in a queue until there are 64 of them (or no node is
+            // left): the expensive part -- fetch the Gaussian, test its ellipsoid, build its table
+            // entry -- then runs with every lane busy, not with the few leaves one step turns up.
+            const int m = S.lqn < 64 ? S.lqn : 64;
+            bool leaf_hit = lane < m;
+            const int32_t left = leaf_hit ? s_leafq[S.lqn - m + lane] : 0;
+            S.lqn -= m;
+            Prim p;
+            f3 U, V, W;
+            float dmin = 0.f, dmax = 0.f;
+            if (leaf_hit) {
+                p = P.prims[~left];
+                quat_to_cols(p.quat4, U, V, W);
+                const f3 O = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
+                // semi-axes of the k-sigma ellipsoid: k * scale = 1 / inv_inter
+                // (bounds only: hardware reciprocal and square root, their last-bit error is inside the 1.001 factors)
+                const f3 ax = mk3(__builtin_amdgcn_rcpf(p.inv_inter4.x), __builtin_amdgcn_rcpf(p.inv_inter4.y), __builtin_amdgcn_rcpf(p.inv_inter4.z));
+                const float dist = __builtin_amdgcn_sqrtf(dot3(O, O));
+                const float amax = fmaxf(ax.x, fmaxf(ax.y, ax.z));
+                const float rad = amax * 1.001f + 1e-5f * dist + F.pad;
+                // Along a ray of direction d the ellipsoid lies within (centre - eye).d -+ |A R^T d|.  For
+                // d = dc that is depth -+ h; a ray at angle <= delta from dc moves the centre term by at
+                // most |depth| delta^2 / 2 + |offset of the centre from the central ray| delta and the
+                // extent by at most amax delta.  The bounding sphere's shell bounds the same range.
+                const float depth = -dot3(O, F.dc);
+                const f3 off = mk3(-O.x - depth * F.dc.x, -O.y - depth * F.dc.y, -O.z - depth * F.dc.z);
+                const float eu = dot3(U, F.dc) * ax.x, ev = dot3(V, F.dc) * ax.y, ew = dot3(W, F.dc) * ax.z;
+                const float ext = __builtin_amdgcn_sqrtf((eu * eu + ev * ev) + ew * ew) * 1.001f;
+                const float slack = 1.5f * (0.5f * fabsf(depth) * F.delta * F.delta + (__builtin_amdgcn_sqrtf(dot3(off, off)) + amax) * F.delta) +
+                                    1e-5f * dist + F.pad;
+                dmin = fmaxf(dist - rad, depth - ext - slack);
+                dmax = fminf(dist + rad, depth + ext + slack);
+                bool ok = p.inv_inter4.w == p.inv_inter4.w; // k is NaN below the density threshold: never hit
+                ok = ok && dmax >= F.t0 && dmin <= F.t1;
+    #pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const f3 n = F.n[k];
+                    // the ellipsoid reaches h beyond its centre along n; centre - eye = -O
+                    const float hu = dot3(U, n) * ax.x, hv = dot3(V, n) * ax.y, hw = dot3(W, n) * ax.z;
+                    const float h = __builtin_amdgcn_sqrtf((hu * hu + hv * hv) + hw * hw) * 1.001f;
+                    ok = ok && !(-dot3(n, O) - h > F.pad);
+                }
+                leaf_hit = ok;
+            }
+            const uint64_t bl = __ballot(leaf_hit);
+            if (leaf_hit) {
+                float4 *dst = (float4 *)(s_tab + (C + __popcll(bl & lt)) * RGX_TAB);
+                const f3 inv = mk3(p.inv_inter4.x, p.inv_inter4.y, p.inv_inter4.z);
+                const f3 O = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
+                dst[0] = make_float4(U.x, U.y, U.z, dmin);
+                dst[1] = make_float4(V.x, V.y, V.z, dmax);
+                dst[2] = make_float4(W.x, W.y, W.z, p.inv_inter4.w);
+                const f3 Oe = apply_sinv_rt(O, U, V, W, inv);
+                dst[3] = make_float4(inv.x, inv.y, inv.z, fmaf(Oe.x, Oe.x, fmaf(Oe.y, Oe.y, fmaf(Oe.z, Oe.z, -1.0f))));
+                dst[4] = make_float4(Oe.x, Oe.y, Oe.z, __int_as_float(~left));
+            }
+            C += __popcll(bl);
+            __syncthreads();
+            continue;
+        }
+        // a step of the descent: up to 64 nodes, one per lane
         const int m = S.qn > RGX_QCAP - RGX_DFS_MARGIN ? 1 : (S.qn < 64 ? S.qn : 64);
         const int base = S.qn - m;
         int32_t node = -1;
@@ -366,57 +430,9 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
             }
         }
         if (lane == 0) cn.nodes += (unsigned)m;
-        // leaf: test the actual ellipsoid, then (after the wave has agreed on table slots) write the entry
-        Prim p;
-        f3 U, V, W;
-        float dmin = 0.f, dmax = 0.f;
-        if (leaf_hit) {
-            p = P.prims[~left];
-            quat_to_cols(p.quat4, U, V, W);
-            const f3 O = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
-            // semi-axes of the k-sigma ellipsoid: k * scale = 1 / inv_inter
-            // (bounds only: hardware reciprocal and square root, their last-bit error is inside the 1.001 factors)
-            const f3 ax = mk3(__builtin_amdgcn_rcpf(p.inv_inter4.x), __builtin_amdgcn_rcpf(p.inv_inter4.y), __builtin_amdgcn_rcpf(p.inv_inter4.z));
-            const float dist = __builtin_amdgcn_sqrtf(dot3(O, O));
-            const float amax = fmaxf(ax.x, fmaxf(ax.y, ax.z));
-            const float rad = amax * 1.001f + 1e-5f * dist + F.pad;
-            // Along a ray of direction d the ellipsoid lies within (centre - eye).d -+ |A R^T d|.  For
-            // d = dc that is depth -+ h; a ray at angle <= delta from dc moves the centre term by at
-            // most |depth| delta^2 / 2 + |offset of the centre from the central ray| delta and the
-            // extent by at most amax delta.  The bounding sphere's shell bounds the same range.
-            const float depth = -dot3(O, F.dc);
-            const f3 off = mk3(-O.x - depth * F.dc.x, -O.y - depth * F.dc.y, -O.z - depth * F.dc.z);
-            const float eu = dot3(U, F.dc) * ax.x, ev = dot3(V, F.dc) * ax.y, ew = dot3(W, F.dc) * ax.z;
-            const float ext = __builtin_amdgcn_sqrtf((eu * eu + ev * ev) + ew * ew) * 1.001f;
-            const float slack = 1.5f * (0.5f * fabsf(depth) * F.delta * F.delta + (__builtin_amdgcn_sqrtf(dot3(off, off)) + amax) * F.delta) +
-                                1e-5f * dist + F.pad;
-            dmin = fmaxf(dist - rad, depth - ext - slack);
-            dmax = fminf(dist + rad, depth + ext + slack);
-            bool ok = p.inv_inter4.w == p.inv_inter4.w; // k is NaN below the density threshold: never hit
-            ok = ok && dmax >= F.t0 && dmin <= F.t1;
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const f3 n = F.n[k];
-                // the ellipsoid reaches h beyond its centre along n; centre - eye = -O
-                const float hu = dot3(U, n) * ax.x, hv = dot3(V, n) * ax.y, hw = dot3(W, n) * ax.z;
-                const float h = __builtin_amdgcn_sqrtf((hu * hu + hv * hv) + hw * hw) * 1.001f;
-                ok = ok && !(-dot3(n, O) - h > F.pad);
-            }
-            leaf_hit = ok;
-        }
         const uint64_t bl = __ballot(leaf_hit), bi = __ballot(inner_hit);
-        if (leaf_hit) {
-            float4 *dst = (float4 *)(s_tab + (C + __popcll(bl & lt)) * RGX_TAB);
-            const f3 inv = mk3(p.inv_inter4.x, p.inv_inter4.y, p.inv_inter4.z);
-            const f3 O = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
-            dst[0] = make_float4(U.x, U.y, U.z, dmin);
-            dst[1] = make_float4(V.x, V.y, V.z, dmax);
-            dst[2] = make_float4(W.x, W.y, W.z, p.inv_inter4.w);
-            const f3 Oe = apply_sinv_rt(O, U, V, W, inv);
-            dst[3] = make_float4(inv.x, inv.y, inv.z, fmaf(Oe.x, Oe.x, fmaf(Oe.y, Oe.y, fmaf(Oe.z, Oe.z, -1.0f))));
-            dst[4] = make_float4(Oe.x, Oe.y, Oe.z, __int_as_float(~left));
-        }
-        C += __popcll(bl);
+        if (leaf_hit) s_leafq[S.lqn + __popcll(bl & lt)] = left; // fewer than 64 waiting + at most 64 new <= 128
+        S.lqn += __popcll(bl);
         if (inner_hit) {
             const int pos = S.qn + 2 * __popcll(bi & lt);
             if (pos + 1 < RGX_QCAP) { // cannot fail: see RGX_DFS_MARGIN (tree depth < 128)
@@ -428,7 +444,7 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
         if (S.qn > RGX_QCAP) S.qn = RGX_QCAP;
         __syncthreads();
     }
-    done = S.qn == 0;
+    done = S.qn == 0 && S.lqn == 0;
     return C;
 }
 
@@ -599,6 +615,7 @@ __device__ __forceinline__ uint32_t row_or(uint32_t v)
 // ---------------------------------------------------------------------------
 struct TileLds {
     int32_t *queue;        // [RGX_QCAP]
+    int32_t *leafq;        // [128]: leaves waiting for the sweep's ellipsoid test
     float *tab;            // [RGX_CCAP * RGX_TAB]
     uint8_t *rowlist;      // [4][RGX_CCAP]: per 16-lane row, table slots some lane of the row hits
     uint32_t (*mask)[64];  // [RGX_CCAP / 32][64]: per lane, hit bits over its row's list
@@ -1072,7 +1089,7 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
             else lo = wave_min_all(run && tmid < thi ? fmaxf(tlo, tmid) : INFINITY), hi = wave_max_all(run ? thi : -INFINITY);
             if (!(lo <= hi)) break; // no ray reaches into the second half
         }
-        Sweep S = {0};
+        Sweep S = {0, 0};
         if (!reuse) {
             float wend = hi;
             if (!split && phase == 0 && Wn.k > 1)
@@ -1088,7 +1105,7 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                 more = false;
             } else {
                 bool done;
-                C = sweep_next(P, S, F, L.queue, L.tab, done, cn);
+                C = sweep_next(P, S, F, L.queue, L.leafq, L.tab, done, cn);
                 if (split) {
                     seen += C;
                 } else if (phase == 0 && first) {
@@ -1236,11 +1253,12 @@ struct Replayer {
 
 #define RGX_TILE_LDS()                                                \
     __shared__ int32_t s_queue[RGX_QCAP];                             \
+    __shared__ int32_t s_leafq[128];                                  \
     __shared__ __align__(16) float s_tab[RGX_CCAP * RGX_TAB];         \
     __shared__ uint8_t s_rowlist[4 * RGX_CCAP];                       \
     __shared__ uint32_t s_mask[RGX_CCAP / 32][64];                    \
     __shared__ uint32_t s_half[2][4][RGX_CCAP / 32];                  \
-    const TileLds L = {s_queue, s_tab, s_rowlist, s_mask, s_half}
+    const TileLds L = {s_queue, s_leafq, s_tab, s_rowlist, s_mask, s_half}
 
 // lane -> pixel: row r = lane / 16 is the 4x4 block (r & 1, r >> 1) of the 8x8 tile
 __device__ __forceinline__ void lane_pixel(int px0, int py0, int &px, int &py)

@@ -25,7 +25,7 @@
 #include <type_traits>
 
 #ifndef RGX_QCAP
-#define RGX_QCAP 448       // node stack entries per wave (LDS)
+#define RGX_QCAP 400       // node stack entries per wave (LDS)
 #endif
 #ifndef RGX_CCAP
 #define RGX_CCAP 128       // candidate table entries per wave (LDS)

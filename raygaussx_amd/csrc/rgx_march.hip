@@ -945,11 +945,55 @@ struct NoRecorder {
 
 __device__ __forceinline__ uint32_t uni_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
-// The replaying backward keeps, per tile, the gradient sums of the current window's Gaussians in
-// LDS (one column of 14 per table slot): a row's share is added there with LDS atomics, and the
-// sums go to memory once per window instead of once per row, slab and Gaussian.
+// What the backward sums per Gaussian over rays and slabs, 13 words: sum y (d density), the colour
+// gradient (3), sum y (Mx) (3) and the symmetric sum y (Mx)(Mx)^T (xx, yy, zz, xy, xz, yz), where
+// Mx = S^-1 R^T (x - centre) is the sample point in the Gaussian's whitened frame.  Every
+// gradient of the Gaussian is linear in these, so the change of variables below runs once per
+// Gaussian and window (or row), not once per ray.
+#define RGX_NSUM 13
+
+// The 14 gradient words (density, rgb, position, scale, quaternion) from the 13 sums
+// (backward/gaussians_aabb.cu:443-481).
+__device__ __forceinline__ void sums_to_gradients(const Prim *pr, const float *s, float *out)
+{
+    const float4 q4 = pr->quat4, i4 = pr->inv_inter4;
+    const float rho = pr->rgba4.w;
+    f3 U, V, W;
+    quat_to_cols(q4, U, V, W);
+    const f3 inv_s = mk3(i4.x * i4.w, i4.y * i4.w, i4.z * i4.w);
+    const f3 sc = mk3(1.0f / inv_s.x, 1.0f / inv_s.y, 1.0f / inv_s.z);
+    const f3 Us = U * inv_s.x, Vs = V * inv_s.y, Ws = W * inv_s.z; // rows of M
+    const f3 Vy = mk3(s[4], s[5], s[6]);
+    out[0] = s[0];
+    out[1] = s[1]; out[2] = s[2]; out[3] = s[3];
+    // d position = rho M^T sum y (Mx)
+    out[4] = rho * (Us.x * Vy.x + Vs.x * Vy.y + Ws.x * Vy.z);
+    out[5] = rho * (Us.y * Vy.x + Vs.y * Vy.y + Ws.y * Vy.z);
+    out[6] = rho * (Us.z * Vy.x + Vs.z * Vy.y + Ws.z * Vy.z);
+    // d scale_a = rho sum y (Mx)_a^2 / scale_a
+    out[7] = rho * s[7] * inv_s.x; out[8] = rho * s[8] * inv_s.y; out[9] = rho * s[9] * inv_s.z;
+    // Q_a = sum y x (Mx)_a with x = R S (Mx);  d R column a = -rho Q_a / scale_a
+    const f3 Ux = U * sc.x, Vx = V * sc.y, Wx = W * sc.z;
+    const f3 Qx = (Ux * s[7] + Vx * s[10]) + Wx * s[11];
+    const f3 Qy = (Ux * s[10] + Vx * s[8]) + Wx * s[12];
+    const f3 Qz = (Ux * s[11] + Vx * s[12]) + Wx * s[9];
+    const f3 d1 = Qx * (-rho * inv_s.x), d2 = Qy * (-rho * inv_s.y), d3 = Qz * (-rho * inv_s.z);
+    const float qx = q4.x, qy = q4.y, qz = q4.z, qw = q4.w;
+    // backward/gaussians_aabb.cu:469-481
+    out[10] = 2 * qw * d1.y - 2 * qz * d1.z - 2 * qw * d2.x + 2 * qy * d2.z + 2 * qz * d3.x - 2 * qy * d3.y;
+    out[11] = 2 * qz * d1.y + 2 * qw * d1.z + 2 * qz * d2.x - 4 * qy * d2.y + 2 * qx * d2.z + 2 * qw * d3.x - 2 * qx * d3.y -
+              4 * qy * d3.z;
+    out[12] = -4 * qz * d1.x + 2 * qy * d1.y - 2 * qx * d1.z + 2 * qy * d2.x + 2 * qw * d2.z + 2 * qx * d3.x + 2 * qw * d3.y -
+              4 * qz * d3.z;
+    out[13] = -4 * qw * d1.x + 2 * qx * d1.y + 2 * qy * d1.z - 2 * qx * d2.x - 4 * qw * d2.y + 2 * qz * d2.z + 2 * qy * d3.x +
+              2 * qz * d3.y;
+}
+
+// The replaying backward keeps, per tile, the sums of the current window's Gaussians in LDS (one
+// column of RGX_NSUM per table slot): a row's share is added there with LDS atomics, and the
+// gradients go to memory once per window instead of once per row, slab and Gaussian.
 struct ReplayLds {
-    float *acc;        // [14][RGX_CCAP], component-major so that different slots fall in different banks
+    float *acc;        // [RGX_NSUM][RGX_CCAP], component-major so that different slots fall in different banks
     uint32_t *pid;     // [RGX_CCAP]: the window's Gaussians by slot
     uint32_t *touched; // [RGX_CCAP / 32]: slots with something in acc
 };
@@ -959,12 +1003,17 @@ __device__ __forceinline__ void replay_flush(const MarchParams &P, const ReplayL
     __syncthreads();
     for (int slot = threadIdx.x; slot < RGX_CCAP; slot += 64) {
         if ((RL.touched[slot >> 5] >> (slot & 31)) & 1u) {
-            float *dst = P.gbuf + (int64_t)RL.pid[slot] * 16;
+            const int64_t pid = RL.pid[slot];
+            float sums[RGX_NSUM], out[14];
 #pragma unroll
-            for (int c = 0; c < 14; ++c) {
-                unsafeAtomicAdd(dst + c, RL.acc[c * RGX_CCAP + slot]);
+            for (int c = 0; c < RGX_NSUM; ++c) {
+                sums[c] = RL.acc[c * RGX_CCAP + slot];
                 RL.acc[c * RGX_CCAP + slot] = 0.f;
             }
+            sums_to_gradients(P.prims + pid, sums, out);
+            float *dst = P.gbuf + pid * 16;
+#pragma unroll
+            for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, out[c]);
         }
     }
     __syncthreads();
@@ -1428,11 +1477,11 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
         if (record_usable(P, reg)) return; // replayed
     }
     const int lane = threadIdx.x;
-    __shared__ float s_acc[REPLAY ? 14 * RGX_CCAP : 1];
+    __shared__ float s_acc[REPLAY ? RGX_NSUM * RGX_CCAP : 1];
     __shared__ uint32_t s_pid[REPLAY ? RGX_CCAP : 1], s_touched[REPLAY ? RGX_CCAP / 32 : 1];
     const ReplayLds RL = {s_acc, s_pid, s_touched};
     if constexpr (REPLAY) {
-        for (int i = lane; i < 14 * RGX_CCAP; i += 64) s_acc[i] = 0.f;
+        for (int i = lane; i < RGX_NSUM * RGX_CCAP; i += 64) s_acc[i] = 0.f;
         for (int i = lane; i < RGX_CCAP; i += 64) s_pid[i] = 0u;
         if (lane < RGX_CCAP / 32) s_touched[lane] = 0u;
         __syncthreads();
@@ -1515,11 +1564,10 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                 return has;
             };
             // (3) per table entry: moments per lane, row sum, one set of atomics per row
-            const f3 xdir_c = dir * fmaf(dt, 16.0f, tbuffer); // slab centre: t_c = tbuffer + 16 dt
             auto gradients = [&](const auto &e, bool hit, bool live, auto) {
-                float out[14];
+                float out[RGX_NSUM];
 #pragma unroll
-                for (int c = 0; c < 14; ++c) out[c] = 0.f;
+                for (int c = 0; c < RGX_NSUM; ++c) out[c] = 0.f;
                 const int32_t pid = e.pid;
                 if (hit) {
                     const Prim *pr = e.prim;
@@ -1557,54 +1605,39 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                         power += inc;
                         inc += inc_st;
                     }
-                    // moments -> gradients.  x_k = xc + u_k dt dir, (Mx)_k = Mxc + u_k dt Md
-                    const f3 xc = prel + xdir_c;
-                    const f3 Mxc = (M1 * xc.x + M2 * xc.y) + M3 * xc.z;
+                    // moments -> sums in the whitened frame.  (Mx)_k = Mxc + u_k dt Md, Mxc at the slab centre (u = 0)
+                    const f3 Mxc = Mx0 + Md * (15.5f * dt);
                     const float m1 = s1 * dt, m2 = s2 * (dt * dt);
-                    const f3 Vy = Mxc * s0 + Md * m1; // sum y (Mx)
-                    const f3 Sy = mk3(fmaf(Mxc.x * Mxc.x, s0, fmaf(2.0f * Mxc.x * Md.x, m1, Md.x * Md.x * m2)),
-                                      fmaf(Mxc.y * Mxc.y, s0, fmaf(2.0f * Mxc.y * Md.y, m1, Md.y * Md.y * m2)),
-                                      fmaf(Mxc.z * Mxc.z, s0, fmaf(2.0f * Mxc.z * Md.z, m1, Md.z * Md.z * m2))); // sum y (Mx)_a^2
-                    // Q_a = sum y x (Mx)_a  (one vector per row a of M)
-                    const f3 Qx = (xc * (Mxc.x * s0) + (xc * Md.x + dir * Mxc.x) * m1) + dir * (Md.x * m2);
-                    const f3 Qy = (xc * (Mxc.y * s0) + (xc * Md.y + dir * Mxc.y) * m1) + dir * (Md.y * m2);
-                    const f3 Qz = (xc * (Mxc.z * s0) + (xc * Md.z + dir * Mxc.z) * m1) + dir * (Md.z * m2);
-                    out[0] = s0; // d density
+                    // sum y (Mx) = B;  sum y (Mx)_a (Mx)_b = Mxc_a B_b + Md_a E_b
+                    const f3 B = Mxc * s0 + Md * m1, E = Mxc * m1 + Md * m2;
                     const float gcol = gc * rho;
-                    out[1] = g.x * gcol; out[2] = g.y * gcol; out[3] = g.z * gcol;                         // d rgb
-                    out[4] = rho * dot3(M1, Vy); out[5] = rho * dot3(M2, Vy); out[6] = rho * dot3(M3, Vy); // d position
-                    out[7] = rho * Sy.x * inv_s.x; out[8] = rho * Sy.y * inv_s.y; out[9] = rho * Sy.z * inv_s.z; // d scale
-                    const f3 d1 = Qx * (-rho * inv_s.x), d2 = Qy * (-rho * inv_s.y), d3 = Qz * (-rho * inv_s.z); // d R columns
-                    const float4 q4 = pr->quat4;
-                    const float qx = q4.x, qy = q4.y, qz = q4.z, qw = q4.w;
-                    // backward/gaussians_aabb.cu:469-481
-                    out[10] = 2 * qw * d1.y - 2 * qz * d1.z - 2 * qw * d2.x + 2 * qy * d2.z + 2 * qz * d3.x - 2 * qy * d3.y;
-                    out[11] = 2 * qz * d1.y + 2 * qw * d1.z + 2 * qz * d2.x - 4 * qy * d2.y + 2 * qx * d2.z + 2 * qw * d3.x -
-                              2 * qx * d3.y - 4 * qy * d3.z;
-                    out[12] = -4 * qz * d1.x + 2 * qy * d1.y - 2 * qx * d1.z + 2 * qy * d2.x + 2 * qw * d2.z + 2 * qx * d3.x +
-                              2 * qw * d3.y - 4 * qz * d3.z;
-                    out[13] = -4 * qw * d1.x + 2 * qx * d1.y + 2 * qy * d1.z - 2 * qx * d2.x - 4 * qw * d2.y + 2 * qz * d2.z +
-                              2 * qy * d3.x + 2 * qz * d3.y;
+                    out[0] = s0;
+                    out[1] = g.x * gcol; out[2] = g.y * gcol; out[3] = g.z * gcol;
+                    out[4] = B.x; out[5] = B.y; out[6] = B.z;
+                    out[7] = fmaf(Mxc.x, B.x, Md.x * E.x);
+                    out[8] = fmaf(Mxc.y, B.y, Md.y * E.y);
+                    out[9] = fmaf(Mxc.z, B.z, Md.z * E.z);
+                    out[10] = fmaf(Mxc.x, B.y, Md.x * E.y);
+                    out[11] = fmaf(Mxc.x, B.z, Md.x * E.z);
+                    out[12] = fmaf(Mxc.y, B.z, Md.y * E.z);
                 }
-                if constexpr (REPLAY) {
-                    // summed over the row's rays, one lane per row adds to the window's sums in LDS
-                    const uint64_t bal = __ballot(hit);
+                // summed over the row's rays; one lane per row carries the sums on
+                const uint64_t bal = __ballot(hit);
 #pragma unroll
-                    for (int c = 0; c < 14; ++c) out[c] = row_sum(out[c]);
-                    if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
+                for (int c = 0; c < RGX_NSUM; ++c) out[c] = row_sum(out[c]);
+                if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
+                    if constexpr (REPLAY) {
+                        // to the window's sums in LDS
                         atomicOr(&s_touched[e.slot >> 5], 1u << (e.slot & 31));
 #pragma unroll
-                        for (int c = 0; c < 14; ++c) unsafeAtomicAdd(&s_acc[c * RGX_CCAP + e.slot], out[c]);
-                    }
-                } else {
-                    // summed over the row's rays, one lane per row adds to memory
-                    const uint64_t bal = __ballot(hit);
-#pragma unroll
-                    for (int c = 0; c < 14; ++c) out[c] = row_sum(out[c]);
-                    if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
+                        for (int c = 0; c < RGX_NSUM; ++c) unsafeAtomicAdd(&s_acc[c * RGX_CCAP + e.slot], out[c]);
+                    } else {
+                        // to memory
+                        float grad[14];
+                        sums_to_gradients(e.prim, out, grad);
                         float *dst = P.gbuf + (int64_t)pid * 16;
 #pragma unroll
-                        for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, out[c]);
+                        for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, grad[c]);
                     }
                 }
             };

@@ -132,7 +132,10 @@ int rgx_pack_prims(const void *ws, const float *eye, const float *pos, const flo
 
 /* ---- ray march ------------------------------------------------------------ */
 
-/* Scratch for one march launch: the backward's Morton-ordered gradient block.  (The
+/* Scratch for one march launch: the backward's Morton-ordered gradient block (64 bytes per
+ * Gaussian) and, sized from n_rays, the order in which the replaying backward takes the image's
+ * tiles (largest hit-list record first).  A workspace that only has room for the gradient block
+ * (64 n bytes rounded up to 256) is accepted: the tiles then run in launch order.  (The
  * reference's per-ray hit scratch hit_prim_idx, optix_utils.py:306, has no counterpart.) */
 int rgx_march_workspace_bytes(int64_t n, int64_t n_rays, int32_t max_prim_slice, size_t *bytes);
 

@@ -57,6 +57,8 @@ struct MarchParams {
     uint32_t *records;      // hit-list record stream, rec_tile_words per tile, or null
     int32_t rec_tile_words;
     int32_t only_overflow;  // backward: handle only the tiles whose record overflowed
+    uint32_t *tile_order;   // per XCD, its list positions from the heaviest tile to the lightest (or null: as launched)
+    int32_t use_tile_order;
 };
 
 struct Counters {
@@ -472,9 +474,12 @@ __host__ __device__ __forceinline__ TileGrid tile_grid(int tiles_x, int tiles_y)
 __device__ __forceinline__ bool tile_origin(const MarchParams &P, int &px0, int &py0, int *tile_out = nullptr)
 {
     const TileGrid g = tile_grid(P.tiles_x, P.tiles_y);
-    const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+    const int xcd = blockIdx.x & 7;
     const int per_block = g.bw * RGX_BLOCK_H;
-    const int block = xcd + 8 * (j / per_block), within = j % per_block;
+    int j = blockIdx.x >> 3;
+    if (P.use_tile_order) j = (int)P.tile_order[xcd * (g.per_xcd * per_block) + j];
+    int block = xcd + 8 * (j / per_block);
+    const int within = j % per_block;
     const int tx = (block % g.blocks_x) * g.bw + within % g.bw;
     const int ty = (block / g.blocks_x) * RGX_BLOCK_H + within / g.bw;
     px0 = tx * 8;
@@ -646,11 +651,11 @@ __device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, f
 }
 
 // A Gaussian as the shading code sees it: its record in HBM plus its rotation columns,
-// inverse scales / k and k -- read from the LDS table entry when there is one, recomputed
-// from the record (same operations, same values) when a recorded hit list is replayed.
+// inverse scales / k and k -- read from the LDS table entry when there is one, from the packed
+// 12-word frame (same operations, same values) that the replay keeps per window slot otherwise.
 template <bool FROM_TABLE>
 struct Entry {
-    const float4 *tab; // LDS table entry (FROM_TABLE only)
+    const float4 *tab; // LDS table entry (FROM_TABLE), or the replay's 3-word frame of the slot
     const Prim *prim;
     int32_t pid;       // index in Morton order
     int slot;          // its slot in the candidate table of the current window
@@ -662,10 +667,10 @@ struct Entry {
             inv = mk3(e3.x, e3.y, e3.z);
             k = e2.w;
         } else {
-            const float4 q = prim->quat4, i4 = prim->inv_inter4;
-            quat_to_cols(q, U, V, W);
-            inv = mk3(i4.x, i4.y, i4.z);
-            k = i4.w;
+            const float4 f0 = tab[0], f1 = tab[1], f2 = tab[2];
+            U = mk3(f0.x, f0.y, f0.z); V = mk3(f0.w, f1.x, f1.y); W = mk3(f1.z, f1.w, f2.x);
+            inv = mk3(f2.y, f2.z, f2.w);
+            k = prim->inv_inter4.w;
         }
     }
 };
@@ -992,18 +997,21 @@ __device__ __forceinline__ void sums_to_gradients(const Prim *pr, const float *s
 // The replaying backward keeps, per tile, the sums of the current window's Gaussians in LDS (one
 // column of RGX_NSUM per table slot): a row's share is added there with LDS atomics, and the
 // gradients go to memory once per window instead of once per row, slab and Gaussian.
+#define RGX_SLOT_TOUCHED 0x80000000u
 struct ReplayLds {
     float *acc;        // [RGX_NSUM][RGX_CCAP], component-major so that different slots fall in different banks
-    uint32_t *pid;     // [RGX_CCAP]: the window's Gaussians by slot
-    uint32_t *touched; // [RGX_CCAP / 32]: slots with something in acc
+    uint32_t *pid;     // [RGX_CCAP]: the window's Gaussians by slot; top bit: the slot has something in acc
+    float4 *frame;     // [RGX_CCAP][3]: rotation columns U, V, W and (1/scale)/k of the window's Gaussians
 };
 
 __device__ __forceinline__ void replay_flush(const MarchParams &P, const ReplayLds &RL)
 {
     __syncthreads();
     for (int slot = threadIdx.x; slot < RGX_CCAP; slot += 64) {
-        if ((RL.touched[slot >> 5] >> (slot & 31)) & 1u) {
-            const int64_t pid = RL.pid[slot];
+        const uint32_t word = RL.pid[slot];
+        if (word & RGX_SLOT_TOUCHED) {
+            const int64_t pid = word & ~RGX_SLOT_TOUCHED;
+            RL.pid[slot] = (uint32_t)pid;
             float sums[RGX_NSUM], out[14];
 #pragma unroll
             for (int c = 0; c < RGX_NSUM; ++c) {
@@ -1017,8 +1025,6 @@ __device__ __forceinline__ void replay_flush(const MarchParams &P, const ReplayL
         }
     }
     __syncthreads();
-    if (threadIdx.x < RGX_CCAP / 32) RL.touched[threadIdx.x] = 0u;
-    __syncthreads();
 }
 
 // Makes the WINDOW item at `at` the current window (sums of the previous one go to memory first).
@@ -1027,7 +1033,17 @@ __device__ __forceinline__ void replay_window(const MarchParams &P, const Replay
     if (at == win_at) return;
     replay_flush(P, RL);
     const int C = (int)(uni_u32(reg[at]) & 0xffffu);
-    for (int i = threadIdx.x; i < C && i < RGX_CCAP; i += 64) RL.pid[i] = min(reg[at + 4 + i], (uint32_t)(P.n - 1));
+    for (int i = threadIdx.x; i < C && i < RGX_CCAP; i += 64) {
+        const uint32_t pid = min(reg[at + 4 + i], (uint32_t)(P.n - 1));
+        RL.pid[i] = pid;
+        const Prim *pr = P.prims + pid;
+        const float4 i4 = pr->inv_inter4;
+        f3 U, V, W;
+        quat_to_cols(pr->quat4, U, V, W);
+        RL.frame[3 * i] = make_float4(U.x, U.y, U.z, V.x);
+        RL.frame[3 * i + 1] = make_float4(V.y, V.z, W.x, W.y);
+        RL.frame[3 * i + 2] = make_float4(W.z, i4.x, i4.y, i4.z);
+    }
     win_at = at;
     __syncthreads();
 }
@@ -1063,8 +1079,8 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
                 slot = slots[w * 32 + __builtin_ctz(bits)] & (RGX_CCAP - 1);
                 bits &= bits - 1u;
             }
-            const int32_t pid = (int32_t)RL.pid[slot];
-            body(Entry<false>{nullptr, P.prims + pid, pid, slot}, has, has, Half<(WALK & 1)>{});
+            const int32_t pid = (int32_t)(RL.pid[slot] & ~RGX_SLOT_TOUCHED);
+            body(Entry<false>{RL.frame + 3 * slot, P.prims + pid, pid, slot}, has, has, Half<(WALK & 1)>{});
         }
     } else {
         const int maxlen = min(max(max(l0, l1), max(l2, l3)), nw * 32);
@@ -1076,8 +1092,8 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
             if (COUNT && hit) ++p0;
             if (__ballot(hit)) {
                 const int slot = live ? slots[i] & (RGX_CCAP - 1) : 0;
-                const int32_t pid = (int32_t)RL.pid[slot];
-                body(Entry<false>{nullptr, P.prims + pid, pid, slot}, hit, live, Half<0>{});
+                const int32_t pid = (int32_t)(RL.pid[slot] & ~RGX_SLOT_TOUCHED);
+                body(Entry<false>{RL.frame + 3 * slot, P.prims + pid, pid, slot}, hit, live, Half<0>{});
             }
         }
     }
@@ -1478,12 +1494,12 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
     }
     const int lane = threadIdx.x;
     __shared__ float s_acc[REPLAY ? RGX_NSUM * RGX_CCAP : 1];
-    __shared__ uint32_t s_pid[REPLAY ? RGX_CCAP : 1], s_touched[REPLAY ? RGX_CCAP / 32 : 1];
-    const ReplayLds RL = {s_acc, s_pid, s_touched};
+    __shared__ uint32_t s_pid[REPLAY ? RGX_CCAP : 1];
+    __shared__ float4 s_frame[REPLAY ? 3 * RGX_CCAP : 1];
+    const ReplayLds RL = {s_acc, s_pid, s_frame};
     if constexpr (REPLAY) {
         for (int i = lane; i < RGX_NSUM * RGX_CCAP; i += 64) s_acc[i] = 0.f;
         for (int i = lane; i < RGX_CCAP; i += 64) s_pid[i] = 0u;
-        if (lane < RGX_CCAP / 32) s_touched[lane] = 0u;
         __syncthreads();
     }
     int px, py;
@@ -1628,7 +1644,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                 if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
                     if constexpr (REPLAY) {
                         // to the window's sums in LDS
-                        atomicOr(&s_touched[e.slot >> 5], 1u << (e.slot & 31));
+                        atomicOr(&s_pid[e.slot], RGX_SLOT_TOUCHED);
 #pragma unroll
                         for (int c = 0; c < RGX_NSUM; ++c) unsafeAtomicAdd(&s_acc[c * RGX_CCAP + e.slot], out[c]);
                     } else {
@@ -1675,6 +1691,56 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
         }
     }
     flush_stats(P.stats, cn);
+}
+
+// Launch order of the replaying backward.  A tile is one wavefront's work from start to end, so a
+// launch ends with a tail in which ever fewer tiles are still running; the tail is as long as the
+// tiles that start last.  The records say how much work each tile is (words used), so every XCD
+// takes its tiles from the largest record to the smallest and the tail consists of the cheapest
+// tiles.  One workgroup per XCD list: counting sort over 1024 size classes (order within a class
+// does not matter); tiles outside the image and tiles without a usable record go last.
+#define RGX_ORDER_BINS 1024
+__global__ __launch_bounds__(256) void k_tile_order(const MarchParams P)
+{
+    __shared__ uint32_t s_bin[RGX_ORDER_BINS];
+    __shared__ uint32_t s_part[256];
+    const TileGrid g = tile_grid(P.tiles_x, P.tiles_y);
+    const int per_block = g.bw * RGX_BLOCK_H, cnt = g.per_xcd * per_block, xcd = blockIdx.x;
+    auto size_class = [&](int j) -> uint32_t {
+        const int block = xcd + 8 * (j / per_block), within = j % per_block;
+        const int tx = (block % g.blocks_x) * g.bw + within % g.bw;
+        const int ty = (block / g.blocks_x) * RGX_BLOCK_H + within / g.bw;
+        if (tx >= P.tiles_x || ty >= P.tiles_y) return 0u;
+        const uint32_t *reg = P.records + (int64_t)(ty * P.tiles_x + tx) * P.rec_tile_words;
+        if (!record_usable(P, reg)) return 0u;
+        const uint64_t used = min(reg[1], (uint32_t)P.rec_tile_words);
+        return 1u + (uint32_t)(used * (RGX_ORDER_BINS - 2) / (uint32_t)P.rec_tile_words);
+    };
+    for (int i = threadIdx.x; i < RGX_ORDER_BINS; i += 256) s_bin[i] = 0u;
+    __syncthreads();
+    for (int j = threadIdx.x; j < cnt; j += 256) atomicAdd(&s_bin[size_class(j)], 1u);
+    __syncthreads();
+    // first position of each class, classes in descending order: thread t owns classes 4t .. 4t+3
+    const int c0 = 4 * threadIdx.x;
+    const uint32_t n0 = s_bin[c0], n1 = s_bin[c0 + 1], n2 = s_bin[c0 + 2], n3 = s_bin[c0 + 3];
+    s_part[threadIdx.x] = n0 + n1 + n2 + n3;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t run = 0; // tiles in heavier classes
+        for (int t = 255; t >= 0; --t) {
+            const uint32_t c = s_part[t];
+            s_part[t] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+    const uint32_t base = s_part[threadIdx.x];
+    s_bin[c0 + 3] = base;
+    s_bin[c0 + 2] = base + n3;
+    s_bin[c0 + 1] = base + n3 + n2;
+    s_bin[c0] = base + n3 + n2 + n1;
+    __syncthreads();
+    for (int j = threadIdx.x; j < cnt; j += 256) P.tile_order[xcd * cnt + atomicAdd(&s_bin[size_class(j)], 1u)] = (uint32_t)j;
 }
 
 // The backward that searches the tree, and the one that replays the forward's record.  (Three
@@ -1781,21 +1847,26 @@ __global__ __launch_bounds__(64) void k_trace_segments(const MarchParams P, f3 o
 // ---------------------------------------------------------------------------
 static inline dim3 grid_for(int64_t n, int block) { return dim3((unsigned)((n + block - 1) / block)); }
 
+// March workspace: the gradient block (16 words per Gaussian, Morton order) and the tile order of
+// the replaying backward.  The order's room is sized from the ray count alone (images of ordinary
+// proportions fit; a launch whose tile grid needs more runs in launch order).
 struct MarchWs {
-    size_t gbuf, total;
+    size_t gbuf, order, order_words, total;
 };
-static inline MarchWs march_ws_layout(int64_t n)
+static inline MarchWs march_ws_layout(int64_t n, int64_t n_rays)
 {
     MarchWs L;
     L.gbuf = 0;
-    L.total = rgx_align_up((size_t)(n > 0 ? n : 1) * 16 * sizeof(float), 256);
+    L.order = rgx_align_up((size_t)(n > 0 ? n : 1) * 16 * sizeof(float), 256);
+    L.order_words = (size_t)(n_rays / 64) * 5 / 4 + 2048;
+    L.total = L.order + rgx_align_up(L.order_words * sizeof(uint32_t), 256);
     return L;
 }
 
 extern "C" int rgx_march_workspace_bytes(int64_t n, int64_t n_rays, int32_t max_prim_slice, size_t *bytes)
 {
     if (n < 0 || n_rays < 0 || max_prim_slice < 0 || !bytes) return RGX_EINVAL;
-    *bytes = march_ws_layout(n).total;
+    *bytes = march_ws_layout(n, n_rays).total;
     return RGX_OK;
 }
 
@@ -1805,8 +1876,8 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     if (!ws || !cam || !march || n < 0 || (n > 0 && !prims) || cam->width <= 0 || cam->height <= 0 ||
         march->max_prim_slice < 0 || !(march->dt_step > 0.0f) || ((uintptr_t)prims & 15u))
         return RGX_EINVAL;
-    const MarchWs M = march_ws_layout(n);
-    if (!march_ws || march_ws_bytes < M.total || ((uintptr_t)march_ws & 255u)) return RGX_EWORKSPACE;
+    const MarchWs M = march_ws_layout(n, 0);
+    if (!march_ws || march_ws_bytes < M.order || ((uintptr_t)march_ws & 255u)) return RGX_EWORKSPACE;
     const WsLayout L = rgx_ws_layout(n);
     const char *w = (const char *)ws;
     P.cam = *cam;
@@ -1829,6 +1900,11 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     P.records = nullptr;
     P.rec_tile_words = 0;
     P.only_overflow = 0;
+    // room for the tile order?  (a workspace sized for fewer rays, or an image of extreme proportions, goes without)
+    const TileGrid g = tile_grid(P.tiles_x, P.tiles_y);
+    const size_t order_words = (size_t)8 * g.per_xcd * g.bw * RGX_BLOCK_H;
+    P.tile_order = M.order + order_words * sizeof(uint32_t) <= march_ws_bytes ? (uint32_t *)((char *)march_ws + M.order) : nullptr;
+    P.use_tile_order = 0;
     return RGX_OK;
 }
 
@@ -1912,8 +1988,13 @@ extern "C" int rgx_march_backward(const void *ws, const RgxCamera *cam, const Rg
     void *span = rgx_span_begin(RGX_T_MARCH_BWD, s);
     if (P.records) {
         // tiles with a complete record replay it; the few whose record overflowed are recomputed
+        if (P.tile_order) {
+            hipLaunchKernelGGL(k_tile_order, dim3(8), dim3(256), 0, s, P);
+            P.use_tile_order = 1;
+        }
         hipLaunchKernelGGL(k_march_bwd_replay, march_grid(P), dim3(64), 0, s, P);
         P.only_overflow = 1;
+        P.use_tile_order = 0;
     }
     hipLaunchKernelGGL(k_march_bwd, march_grid(P), dim3(64), 0, s, P);
     rgx_span_end(span, s);

@@ -683,6 +683,21 @@ def test_direct_ctypes_binding_matches_the_python_mirror(gx, c0):
                                p(dsh), p(dpos_dir), None, None, None, s) == 0
     dpos += dpos_dir
     torch.cuda.synchronize()
+    # a march workspace with room for the gradient block only (sized for another image, say): the replay
+    # then takes the tiles in launch order instead of heaviest first, and returns the same gradients
+    _step("direct ctypes calls, workspace without room for a tile order")
+    small = (N * 64 + 255) // 256 * 256
+    ddens2, dscale2 = torch.empty_like(ddens), torch.empty_like(dscale)
+    assert lib.rgx_march_backward(p(bvh), C.byref(cam), C.byref(march), p(prims), C.c_int64(N), p(img), p(dimg),
+                                  p(ddens2), p(drgb), p(dpos_dir), p(dscale2), p(dquat), p(mws), C.c_size_t(small),
+                                  p(rec), C.c_size_t(rec.numel()), None, s) == 0
+    torch.cuda.synchronize()
+    for a, b in ((ddens2, ddens), (dscale2, dscale)):
+        cos, rel = gx.cos_rel(a.cpu().numpy(), b.cpu().numpy())
+        assert cos >= 1 - 1e-6 and rel <= 1e-5, (cos, rel)
+    assert lib.rgx_march_backward(p(bvh), C.byref(cam), C.byref(march), p(prims), C.c_int64(N), p(img), p(dimg),
+                                  p(ddens2), p(drgb), p(dpos_dir), p(dscale2), p(dquat), p(mws), C.c_size_t(small - 256),
+                                  p(rec), C.c_size_t(rec.numel()), None, s) == -2   # RGX_EWORKSPACE
     ref = gx.gpu_render(sc, camera, cfg, want_grad=dimg.cpu().numpy(), stats=False)
     np.testing.assert_array_equal(img.cpu().numpy(), ref["image"])
     for name, got in (("positions", dpos), ("scales", dscale), ("quaternions", dquat), ("densities", ddens), ("color_features", dsh)):

@@ -681,6 +681,7 @@ __device__ __forceinline__ float gauss_weight(float power) { return __builtin_am
 // Per-hit constants of the sample recurrence (gaussians_aabb.cu:135-164).
 struct HitSetup {
     float power, inc, inc_st, cut;
+    f3 Mx0, Md; // the first sample point and the ray direction in the Gaussian's whitened frame
 };
 __device__ __forceinline__ HitSetup hit_setup(f3 U, f3 V, f3 W, f3 inv, float k, float4 pos4, f3 dir, f3 ray_dir_tmid, float dt)
 {
@@ -695,6 +696,8 @@ __device__ __forceinline__ HitSetup hit_setup(f3 U, f3 V, f3 W, f3 inv, float k,
     h.inc = Md_dt_2 + 2.0f * dot3(Mx0, Md) * dt;
     h.inc_st = 2.0f * Md_dt_2;
     h.cut = k * k;
+    h.Mx0 = Mx0;
+    h.Md = Md;
     return h;
 }
 
@@ -1478,9 +1481,10 @@ __device__ __forceinline__ float row_sum(float v)
 //   dscale, dpos, dR: sums of y_k times polynomials of degree <= 2 in k, because
 //   the sample point x_k = x_c + u_k dt dir (u_k = k - 15.5) is affine in k.
 // So the inner loop carries three moments (sum y, sum y u, sum y u^2) instead of
-// nineteen running sums; the `power < k^2` mask follows the reference's 32-step
-// recurrence exactly.  The 14 gradient words of a Gaussian are summed over the 16
-// rays of a row with DPP adds before one lane per row adds them to memory.
+// nineteen running sums; the `power < k^2` mask follows the forward's 32-step recurrence, i.e. it
+// is the mask the forward blended with.  Per Gaussian the moments turn into 13 sums in its whitened
+// frame (RGX_NSUM); those are summed over the 16 rays of a row with DPP adds and carried on by one
+// lane per row; the change of variables to the 14 gradient words comes after all sums.
 template <bool REPLAY>
 __device__ __forceinline__ void march_bwd(const MarchParams &P)
 {
@@ -1591,22 +1595,13 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                     f3 U, V, W, inv;
                     float k;
                     e.frame(U, V, W, inv, k);
-                    const f3 inv_s = mk3(inv.x * k, inv.y * k, inv.z * k);
-                    const float cut = k * k;
                     const float rho = col.w;
                     const float dcg = dot3(mk3(col.x, col.y, col.z), g) * __builtin_amdgcn_rcpf(rho);
-                    // mask recurrence exactly as backward/gaussians_aabb.cu:375-396, 437-438
-                    const f3 Us = U * inv_s.x, Vs = V * inv_s.y, Ws = W * inv_s.z;
-                    const f3 M1 = mk3(Us.x, Vs.x, Ws.x), M2 = mk3(Us.y, Vs.y, Ws.y), M3 = mk3(Us.z, Vs.z, Ws.z);
-                    const f3 prel = mk3(e5.x, e5.y, e5.z);
-                    const f3 x0 = prel + dir * (tbuffer + 0.5f * dt);
-                    const f3 Mx0 = (M1 * x0.x + M2 * x0.y) + M3 * x0.z;
-                    const f3 Md = (M1 * dir.x + M2 * dir.y) + M3 * dir.z;
-                    const float Md2 = dot3(Md, Md);
-                    const float Md_dt_2 = (dt * dt) * Md2;
-                    float power = dot3(Mx0, Mx0);
-                    float inc = Md_dt_2 + 2.0f * dot3(Mx0, Md) * dt;
-                    const float inc_st = 2.0f * Md_dt_2;
+                    // the forward's sample recurrence (the mask is the one the forward blended with)
+                    const HitSetup hs = hit_setup(U, V, W, inv, k, e5, dir, rdt0, dt);
+                    const f3 Mx0 = hs.Mx0, Md = hs.Md;
+                    const float cut = hs.cut, inc_st = hs.inc_st;
+                    float power = hs.power, inc = hs.inc;
                     float s0 = 0.f, s1 = 0.f, s2 = 0.f, gc = 0.f;
 #pragma unroll
                     for (int i = 0; i < RGX_BUFFER_SIZE; ++i) {

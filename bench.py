@@ -39,7 +39,7 @@ HBM_PEAK_GBPS = 8000.0
 # script scaled by a 1 GiB copy (--calibrate-copy); the counter readings are kept in
 # profiles/march_kernels_c4_1M_800x800.md.  Workloads without a measurement report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("c4_1M_800x800", "march_backward"): 11.15e9,  # k_march_bwd_replay: 2.9 GB read, 8.3 GB written
+    ("c4_1M_800x800", "march_backward"): 9.43e9,   # k_march_bwd_replay: 2.8 GB read, 6.6 GB written
     ("c4_1M_800x800", "march_forward"): 3.05e9,    # k_march_fwd<true, false>: 1.7 GB read, 1.3 GB written (0.23 the record)
 }
 

@@ -39,8 +39,8 @@ HBM_PEAK_GBPS = 8000.0
 # script scaled by a 1 GiB copy (--calibrate-copy); the counter readings are kept in
 # profiles/march_kernels_c4_1M_800x800.md.  Workloads without a measurement report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("c4_1M_800x800", "march_backward"): 9.43e9,   # k_march_bwd_replay: 2.8 GB read, 6.6 GB written
-    ("c4_1M_800x800", "march_forward"): 3.05e9,    # k_march_fwd<true, false>: 1.7 GB read, 1.3 GB written (0.23 the record)
+    ("c4_1M_800x800", "march_backward"): 19.2e9,   # k_march_bwd_replay_sums: 16.0 GB read (14.0 the sample sums), 3.2 GB written
+    ("c4_1M_800x800", "march_forward"): 20.6e9,    # k_march_fwd<true, false>: 5.4 GB read, 15.2 GB written (14.0 the sample sums)
 }
 
 WORKLOADS = {
@@ -139,6 +139,9 @@ def main():
     ap.add_argument("--forward-only", action="store_true")
     ap.add_argument("--no-records", action="store_true",
                     help="backward searches the tree again instead of replaying the forward's hit-list record")
+    ap.add_argument("--rec-tile-words", type=int, default=None,
+                    help="record size per tile in 32-bit words (16384: hit lists only, no per-sample sums); "
+                         "default: the renderer's own")
     ap.add_argument("--side-kernels", action="store_true",
                     help="time the entry points around the march (image epilogue, reorder gather, distCUDA2, viewer launch) "
                          "instead of the training step; one JSON line")
@@ -146,8 +149,8 @@ def main():
                     help="only run a 1 GiB device-to-device copy (reference reading for the FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU only (--gpus 1); the path shards by views/tiles, "
-                 "see DESIGN.md, but no multi-GPU figure is produced")
+        sys.exit("bench.py: this build measures one GPU only (--gpus 1); the path would shard by views or bands "
+                 "of tiles with one gradient all-reduce per step, but no multi-GPU figure is produced")
     if not torch.cuda.is_available():
         sys.exit("bench.py: needs a GPU (librgx has no CPU path)")
     dev = "cuda:0"
@@ -195,6 +198,8 @@ def main():
                              t_eps=cfg["t_eps"], gas=gas)
         s.stats = stats
         s.record_hits = not args.no_records
+        if args.rec_tile_words is not None:
+            s.rec_tile_words = args.rec_tile_words
         img = RenderOptixFunction.apply(*params, s)
         gas = s.gas
         if not args.forward_only:
@@ -223,18 +228,26 @@ def main():
     mrays = n_rays * args.steps / elapsed / 1e6
     passes = 1 if args.forward_only else 2
     hits_per_launch = st["hit_pairs"] / (args.steps * passes)   # H: fwd and bwd march the same slabs
-    if args.forward_only:
-        kname, alg_bytes = "march_forward", 64.0 * hits_per_launch + 12.0 * n_rays
-    else:
-        kname, alg_bytes = "march_backward", (64.0 + 56.0) * hits_per_launch + 24.0 * n_rays
-    k_ms, k_cnt = timing[kname]
-    k_avg_ms = k_ms / max(k_cnt, 1)
-    achieved = alg_bytes / (k_avg_ms * 1e-3) / 1e9 if k_avg_ms > 0 else 0.0
-    roofline = dict(bound="hbm", kernel="k_march_fwd" if args.forward_only else ("k_march_bwd" if args.no_records else "k_march_bwd_replay"),
-                    achieved=round(achieved, 2), peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBPS, 5),
-                    traffic=None if (args.no_records or args.forward_only) else MEASURED_TRAFFIC_BYTES.get((args.workload, kname)),
-                    kernel_ms=round(k_avg_ms, 4), algorithmic_bytes=int(alg_bytes),
-                    hit_pairs_per_launch=int(hits_per_launch))
+    # the dominant kernel: the march launch (forward or backward) that takes longer
+    bwd_name = "k_march_bwd" if args.no_records else (
+        "k_march_bwd_replay" if (args.rec_tile_words or 1 << 30) < 16384 + 8192 else "k_march_bwd_replay_sums")
+    cand = [("march_forward", "k_march_fwd", 64.0 * hits_per_launch + 12.0 * n_rays)]
+    if not args.forward_only:
+        cand.append(("march_backward", bwd_name, (64.0 + 56.0) * hits_per_launch + 24.0 * n_rays))
+    per_kernel = {}
+    for key, name, nbytes in cand:
+        ms, cnt = timing[key]
+        avg = ms / max(cnt, 1)
+        gbps = nbytes / (avg * 1e-3) / 1e9 if avg > 0 else 0.0
+        per_kernel[key] = dict(kernel=name, kernel_ms=round(avg, 4), algorithmic_bytes=int(nbytes), achieved=round(gbps, 2),
+                               frac=round(gbps / HBM_PEAK_GBPS, 5))
+    kname = max(per_kernel, key=lambda k: per_kernel[k]["kernel_ms"])
+    dom = per_kernel[kname]
+    default_record = not (args.no_records or args.forward_only or args.rec_tile_words is not None)
+    roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=dom["achieved"], peak=HBM_PEAK_GBPS, unit="GB/s", frac=dom["frac"],
+                    traffic=MEASURED_TRAFFIC_BYTES.get((args.workload, kname)) if default_record else None,
+                    kernel_ms=dom["kernel_ms"], algorithmic_bytes=dom["algorithmic_bytes"],
+                    hit_pairs_per_launch=int(hits_per_launch), march_kernels=per_kernel)
     # whole-step roofline-derived rate: all algorithmic bytes of one step at peak bandwidth
     step_bytes = (64.0 * hits_per_launch + 12.0 * n_rays + 300.0 * n
                   + (0 if args.forward_only else (120.0 * hits_per_launch + 24.0 * n_rays + 464.0 * n)))

@@ -139,14 +139,19 @@ int rgx_pack_prims(const void *ws, const float *eye, const float *pos, const flo
  * reference's per-ray hit scratch hit_prim_idx, optix_utils.py:306, has no counterpart.) */
 int rgx_march_workspace_bytes(int64_t n, int64_t n_rays, int32_t max_prim_slice, size_t *bytes);
 
-/* Optional hit-list record of one forward launch: per 8x8 pixel tile a region of tile_words
- * 32-bit words (>= 1024, multiple of 4; 16384 is ample for the benchmark scenes) holding, per
- * slab iteration, which Gaussians each 4x4 pixel row hits and each ray's hit bits.  A backward
- * given the record of its forward replays those lists instead of searching the tree again;
- * tiles whose region overflowed, or whose region was not written by a forward launch with the same
- * number of Gaussians, image size and step, are recomputed.  The role the reference's hit_prim_idx buffer
- * plays between its collect and blend steps (optix_utils.py:306), at a few hundred bytes per
- * tile and slab instead of max_prim_slice ints per ray. */
+/* Optional record of one forward launch, tile_words 32-bit words per 8x8 pixel tile on average
+ * (>= 1024, multiple of 4).  Up to 16384 words per tile hold the hit lists: per slab iteration,
+ * which Gaussians each 4x4 pixel row hits and each ray's hit bits (16384 is ample for the benchmark
+ * scenes).  A backward given the record of its forward replays those lists instead of searching the
+ * tree again; tiles whose region overflowed, or whose region was not written by a forward launch
+ * with the same number of Gaussians, image size and step, are recomputed.  The role the
+ * reference's hit_prim_idx buffer plays between its collect and blend steps (optix_utils.py:306),
+ * at a few hundred bytes per tile and slab instead of max_prim_slice ints per ray.
+ * What tile_words gives beyond 16384 (at least 8192 more) becomes one pool of 32 KiB slots shared
+ * by all tiles: per slab iteration that blends something, the per-sample density and colour sums
+ * of its 64 rays.  The backward then reads these back instead of walking the hit lists once more
+ * to rebuild them (about a fifth faster; 16384 + 64 * 8192 words per tile hold the benchmark
+ * scenes).  Tiles that found the pool empty are replayed from their hit lists alone. */
 int rgx_march_records_bytes(int32_t width, int32_t height, int32_t tile_words, size_t *bytes);
 
 /* Replaces launch_pipeline_forward / launch_pipeline_test (optix_utils.py:222-322,

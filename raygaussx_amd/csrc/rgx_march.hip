@@ -59,6 +59,9 @@ struct MarchParams {
     int32_t only_overflow;  // backward: handle only the tiles whose record overflowed
     uint32_t *tile_order;   // per XCD, its list positions from the heaviest tile to the lightest (or null: as launched)
     int32_t use_tile_order;
+    float4 *sum_pool;       // sample-sum slots of the record (RGX_SUM_SLOT_WORDS each), or null
+    uint32_t *sum_next;     // next free slot (bump counter in the record's pool header)
+    int32_t sum_slots;      // slots in the pool
 };
 
 struct Counters {
@@ -848,13 +851,26 @@ __device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds 
 // iteration.  The forward can stream it to memory so that the backward replays the same lists
 // instead of sweeping the tree and evaluating the predicate again.  Per tile a region of
 // rec_tile_words 32-bit words:
-//   word 0: 0 = complete, 1 = the region overflowed (record unusable);  word 1: words used;
+//   word 0: status (RGX_REC_COMPLETE, _OVERFLOWED, _COMPLETE_SUMS);  word 1: words used;
 //   from word 4, per iteration: WINDOW when a table was built, one LISTS per table, then TRAIL
 //   WINDOW: {tag | C, -, -, -}, pid[pad4(C)]            the table's Gaussians, by slot
 //   LISTS:  {tag | last << 8 | nw, len[4], -, -, -}, slot bytes of row r in pad4(len[r]) / 4 words
 //           for r = 0..3, mask[nw][64], half[2][4][nw]   (the TileLds arrays of the same names;
 //           bytes and words past a row's length are junk)
-//   TRAIL:  {tag | any_search, cover (float), -, -}, found[64] when any_search
+//   TRAIL:  {tag | any_search, cover (float), sample-sum slot + 1, -}, found[64] when any_search
+//
+// Sample sums.  A record with room beyond RGX_REC_LIST_WORDS per tile also has a pool of slots
+// shared by all tiles: per slab iteration that blends something, the per-sample density and colour
+// sums the forward blended -- sum rho w as [32 samples][64 rays], then sum rgb rho w as
+// [32 samples][64 rays][3].  The
+// backward reads them back instead of walking the hit lists a second time to rebuild them.  The
+// iteration's TRAIL item names its slot (word 2: slot + 1, 0 = none).  Tiles take slots from a
+// bump counter; a tile that found the pool empty is marked lists-only (status 0).
+#define RGX_REC_LIST_WORDS 16384   // hit-list words per tile when the record also holds sample sums
+#define RGX_SUM_SLOT_WORDS 8192    // 32 samples x 64 rays x 4 words
+#define RGX_REC_COMPLETE 0u        // word 0 of a tile: hit lists complete
+#define RGX_REC_OVERFLOWED 1u      //   the region overflowed (record unusable)
+#define RGX_REC_COMPLETE_SUMS 2u   //   hit lists and sample sums complete
 #define RGX_REC_WINDOW 0x57000000u
 #define RGX_REC_LISTS 0x4C000000u
 #define RGX_REC_TRAIL 0x54000000u
@@ -866,11 +882,17 @@ __device__ __forceinline__ uint32_t record_mark(const MarchParams &P, int which)
 {
     return which == 0 ? (uint32_t)P.n : ((uint32_t)P.cam.width << 16 ^ (uint32_t)P.cam.height ^ __float_as_uint(P.m.dt_step));
 }
+// Status of a tile's record if it is this launch's and complete, else RGX_REC_OVERFLOWED.
+__device__ __forceinline__ uint32_t record_status(const MarchParams &P, const uint32_t *reg)
+{
+    const uint32_t st = (uint32_t)__builtin_amdgcn_readfirstlane((int)reg[0]);
+    const bool mine = (uint32_t)__builtin_amdgcn_readfirstlane((int)reg[2]) == record_mark(P, 0) &&
+                      (uint32_t)__builtin_amdgcn_readfirstlane((int)reg[3]) == record_mark(P, 1);
+    return mine && (st == RGX_REC_COMPLETE || (st == RGX_REC_COMPLETE_SUMS && P.sum_pool)) ? st : RGX_REC_OVERFLOWED;
+}
 __device__ __forceinline__ bool record_usable(const MarchParams &P, const uint32_t *reg)
 {
-    return (uint32_t)__builtin_amdgcn_readfirstlane((int)reg[0]) == 0u &&
-           (uint32_t)__builtin_amdgcn_readfirstlane((int)reg[2]) == record_mark(P, 0) &&
-           (uint32_t)__builtin_amdgcn_readfirstlane((int)reg[3]) == record_mark(P, 1);
+    return record_status(P, reg) != RGX_REC_OVERFLOWED;
 }
 
 struct Recorder {
@@ -878,6 +900,8 @@ struct Recorder {
     int off;        // next free word (wave-uniform)
     int cap;        // words in the region
     bool ovf;       // the region is exhausted
+    bool sums;      // every blending iteration so far got a sample-sum slot
+    int slot;       // the current iteration's sample-sum slot, or -1
     __device__ __forceinline__ bool on() const { return reg != nullptr && !ovf; }
     // room for an item and the iteration's trailer?
     __device__ __forceinline__ bool fits(int size)
@@ -920,13 +944,23 @@ struct Recorder {
         off += size;
     }
 
-    __device__ __forceinline__ void write_trailer(bool any_search, float cover, float found)
+    // blends: some ray of the wave has hits to blend in this iteration
+    __device__ __forceinline__ void write_trailer(const MarchParams &P, bool any_search, float cover, float found, bool blends)
     {
+        slot = -1;
         if (!on()) return;
+        if (blends && sums) {
+            uint32_t s = 0;
+            if (threadIdx.x == 0) s = atomicAdd(P.sum_next, 1u);
+            s = (uint32_t)__builtin_amdgcn_readfirstlane((int)s);
+            if (s < (uint32_t)P.sum_slots) slot = (int)s;
+            else sums = false;
+        }
         uint32_t *it = reg + off;
         if (threadIdx.x == 0) {
             it[0] = RGX_REC_TRAIL | (any_search ? 1u : 0u);
             it[1] = __float_as_uint(cover);
+            it[2] = (uint32_t)(slot + 1);
         }
         if (any_search) it[4 + threadIdx.x] = __float_as_uint(found);
         off += 4 + (any_search ? 64 : 0);
@@ -935,7 +969,7 @@ struct Recorder {
     __device__ __forceinline__ void finish(const MarchParams &P)
     {
         if (reg && threadIdx.x == 0) {
-            reg[0] = ovf ? 1u : 0u;
+            reg[0] = ovf ? RGX_REC_OVERFLOWED : (sums ? RGX_REC_COMPLETE_SUMS : RGX_REC_COMPLETE);
             reg[1] = (uint32_t)off;
             reg[2] = record_mark(P, 0);
             reg[3] = record_mark(P, 1);
@@ -947,7 +981,8 @@ struct Recorder {
 struct NoRecorder {
     __device__ __forceinline__ void write_window(const TileLds &, int) {}
     __device__ __forceinline__ void write_lists(const TileLds &, int, bool) {}
-    __device__ __forceinline__ void write_trailer(bool, float, float) {}
+    static constexpr int slot = -1;
+    __device__ __forceinline__ void write_trailer(const MarchParams &, bool, float, float, bool) {}
     __device__ __forceinline__ void finish(const MarchParams &) {}
 };
 
@@ -1053,8 +1088,8 @@ __device__ __forceinline__ void replay_window(const MarchParams &P, const Replay
 
 // Replays one LISTS item.  WALK_ROWS: as shade_rows (the four rows walk their recorded lists in lock
 // step); WALK 0 / 1: as shade_lanes over one half's entries; WALK_LANES_ALL: every ray walks all
-// its hits.  COUNT adds the lane's hits to p0.  Returns the item's size.
-enum { WALK_LANES_ALL = 2, WALK_ROWS_ALL = 3 };
+// its hits; WALK_NONE: no walk.  COUNT adds the lane's hits to p0.  Returns the item's size.
+enum { WALK_LANES_ALL = 2, WALK_ROWS_ALL = 3, WALK_NONE = 4 };
 template <bool COUNT, int WALK, typename Body>
 __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLds &RL, const uint32_t *it, bool run, int &p0, Body body)
 {
@@ -1065,7 +1100,11 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
     const int len = row == 0 ? l0 : row == 1 ? l1 : row == 2 ? l2 : l3;
     const uint8_t *slots = (const uint8_t *)(it + 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0));
     const uint32_t *masks = it + 8 + q0 + q1 + q2 + q3 + lane; // word w of this lane: masks[w * 64]
-    if constexpr (WALK != WALK_ROWS_ALL) {
+    if constexpr (WALK == WALK_NONE) {
+        const int nwr = run ? min((len + 31) >> 5, nw) : 0;
+        if (COUNT)
+            for (int w = 0; w < nwr; ++w) p0 += __popc(masks[w * 64]);
+    } else if constexpr (WALK != WALK_ROWS_ALL) {
         const int nwr = run ? min((len + 31) >> 5, nw) : 0; // words of this lane's row; later words are not its own
         const uint32_t *half = it + 8 + q0 + q1 + q2 + q3 + nw * 64 + ((WALK & 1) * 4 + row) * nw;
         auto word = [&](int w) { return WALK == WALK_LANES_ALL ? masks[w * 64] : masks[w * 64] & half[w]; };
@@ -1237,7 +1276,7 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
             }
         }
         if (phase == 0) {
-            rec.write_trailer(any_search, split ? hi : (Wn.resident ? Wn.hi : t1), found);
+            rec.write_trailer(P, any_search, split ? hi : (Wn.resident ? Wn.hi : t1), found, __any(need && p0 > 0));
             run = mid(split);
             if (!__any(run)) break;
         }
@@ -1265,7 +1304,8 @@ struct Replayer {
 
     // The backward's iteration driven by the record instead of the tree: body_a per ray over the
     // recorded lists, once per half of the samples; mid(); body_b over the lists row by row.
-    template <typename BodyA, typename Mid, typename BodyB>
+    // SUMS: body_a(slot) reads the iteration's sample sums instead of walking the lists for them
+    template <bool SUMS, typename BodyA, typename Mid, typename BodyB>
     __device__ __forceinline__ bool slab(const MarchParams &P, const RayState &R, bool need, int &p0, float &found,
                                          float &searched_to, BodyA body_a, Mid mid, BodyB body_b)
     {
@@ -1289,14 +1329,36 @@ struct Replayer {
             return false;
         }
         int dummy = 0;
-        for (int a = start; a < end;) {
-            const uint32_t head = uni_u32(reg[a]);
-            if ((head & 0xff000000u) == RGX_REC_WINDOW) {
-                replay_window(P, RL, reg, a, win_at);
-                a += 4 + (((int)(head & 0xffffu) + 3) & ~3);
-            } else {
-                replay_lists<true, 0>(P, RL, reg + a, need, p0, body_a);
-                a += replay_lists<false, 1>(P, RL, reg + a, need, dummy, body_a);
+        if constexpr (SUMS) {
+            auto none = [](const auto &, bool, bool, auto) {};
+            for (int a = start; a < end;) {
+                const uint32_t head = uni_u32(reg[a]);
+                if ((head & 0xff000000u) == RGX_REC_WINDOW) {
+                    replay_window(P, RL, reg, a, win_at); // later iterations of the window carry no WINDOW item
+                    a += 4 + (((int)(head & 0xffffu) + 3) & ~3);
+                } else {
+                    a += replay_lists<true, WALK_NONE>(P, RL, reg + a, need, p0, none);
+                }
+            }
+            if (__any(need && p0 > 0)) {
+                const uint32_t slot1 = uni_u32(reg[end + 2]);
+                if (slot1 == 0u || slot1 > (uint32_t)P.sum_slots) {
+                    lost = true;
+                    mid(false);
+                    return false;
+                }
+                body_a(P.sum_pool + (int64_t)(slot1 - 1u) * (RGX_SUM_SLOT_WORDS / 4));
+            }
+        } else {
+            for (int a = start; a < end;) {
+                const uint32_t head = uni_u32(reg[a]);
+                if ((head & 0xff000000u) == RGX_REC_WINDOW) {
+                    replay_window(P, RL, reg, a, win_at);
+                    a += 4 + (((int)(head & 0xffffu) + 3) & ~3);
+                } else {
+                    replay_lists<true, 0>(P, RL, reg + a, need, p0, body_a);
+                    a += replay_lists<false, 1>(P, RL, reg + a, need, dummy, body_a);
+                }
             }
         }
         const float cover = __uint_as_float(uni_u32(reg[end + 1]));
@@ -1356,7 +1418,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
     int px0, py0, tile;
     if (!tile_origin(P, px0, py0, &tile)) return; // whole wave
     typename std::conditional<RECORD, Recorder, NoRecorder>::type rec;
-    if constexpr (RECORD) rec = Recorder{P.records + (int64_t)tile * P.rec_tile_words, 4, P.rec_tile_words, false};
+    if constexpr (RECORD) rec = Recorder{P.records + (int64_t)tile * P.rec_tile_words, 4, P.rec_tile_words, false, P.sum_pool != nullptr, -1};
     int px, py;
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
@@ -1420,9 +1482,28 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
                     R.T *= w;
                 }
             };
+            // the chunk's sums go to the iteration's sample-sum slot, if it has one
+            auto keep_sums = [&](int first_sample) {
+                if constexpr (RECORD) {
+                    if (rec.slot >= 0) {
+                        float *slot = (float *)(P.sum_pool + (int64_t)rec.slot * (RGX_SUM_SLOT_WORDS / 4));
+                        float *dens = slot + first_sample * 64 + threadIdx.x;
+                        float *col = slot + RGX_BUFFER_SIZE * 64 + (first_sample * 64 + threadIdx.x) * 3;
+#pragma unroll
+                        for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
+                            // written once, read once by the backward: keep them out of the caches' way
+                            __builtin_nontemporal_store(sg[i], dens + i * 64);
+                            __builtin_nontemporal_store(cr[i], col + i * 192);
+                            __builtin_nontemporal_store(cg[i], col + i * 192 + 1);
+                            __builtin_nontemporal_store(cb[i], col + i * 192 + 2);
+                        }
+                    }
+                }
+            };
             auto second_half = [&](bool split) { // split: the hits of the second half are not known yet
                 const bool has = need && (p0 > 0 || split);
                 if (has) blend();
+                keep_sums(0);
                 // samples 16..31, only for rays still above the transmittance floor (gaussians_aabb.cu:190)
 #pragma unroll
                 for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
@@ -1432,6 +1513,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
             const bool run2 = slab_tables<WALK_FORWARD>(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, accumulate,
                                           second_half, accumulate);
             if (run2) blend();
+            keep_sums(RGX_CHUNK_SIZE);
             if (need && p0 > 0) {
                 cn.slabs++;
                 cn.hit_pairs += p0;
@@ -1485,14 +1567,16 @@ __device__ __forceinline__ float row_sum(float v)
 // is the mask the forward blended with.  Per Gaussian the moments turn into 13 sums in its whitened
 // frame (RGX_NSUM); those are summed over the 16 rays of a row with DPP adds and carried on by one
 // lane per row; the change of variables to the 14 gradient words comes after all sums.
-template <bool REPLAY>
+template <bool REPLAY, bool SUMS>
 __device__ __forceinline__ void march_bwd(const MarchParams &P)
 {
+    static_assert(REPLAY || !SUMS, "sample sums come with a record");
     int px0, py0, tile;
     if (!tile_origin(P, px0, py0, &tile)) return; // whole wave
     const uint32_t *reg = P.records ? P.records + (int64_t)tile * P.rec_tile_words : nullptr;
     if (REPLAY) {
-        if (!record_usable(P, reg)) return; // overflowed, or not this launch's: the other kernel handles the tile
+        // overflowed, not this launch's, or with / without sample sums: another kernel handles the tile
+        if (record_status(P, reg) != (SUMS ? RGX_REC_COMPLETE_SUMS : RGX_REC_COMPLETE)) return;
     } else if (P.only_overflow) {
         if (record_usable(P, reg)) return; // replayed
     }
@@ -1557,6 +1641,17 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                         hs.inc += hs.inc_st;
                     }
                 }
+            };
+            // (1') the same from the forward's sample sums: PA = sum rho w, PB = g . sum rgb rho w
+            auto load_sums = [&](const float4 *slot) {
+                const float *dens = (const float *)slot + lane;
+                const float *col = (const float *)slot + RGX_BUFFER_SIZE * 64 + lane * 3;
+#pragma unroll
+                for (int i = 0; i < RGX_BUFFER_SIZE; ++i) PA[i] = __builtin_nontemporal_load(dens + i * 64);
+#pragma unroll
+                for (int i = 0; i < RGX_BUFFER_SIZE; ++i)
+                    PB[i] = fmaf(g.x, __builtin_nontemporal_load(col + i * 192),
+                                 fmaf(g.y, __builtin_nontemporal_load(col + i * 192 + 1), g.z * __builtin_nontemporal_load(col + i * 192 + 2)));
             };
             // (2) prefix: PA <- a_k, PB <- (T_k e_k - D_k) dt - a_k e_k   (so X_k = PB + PA * g.c_i);
             // it always covers all 32 samples (330-352)
@@ -1652,7 +1747,9 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                     }
                 }
             };
-            const bool has = drive(need, tlo, thi, p0, ov, found, searched_to, densities, prefix, gradients);
+            bool has;
+            if constexpr (SUMS) has = drive(need, tlo, thi, p0, ov, found, searched_to, load_sums, prefix, gradients);
+            else has = drive(need, tlo, thi, p0, ov, found, searched_to, densities, prefix, gradients);
             if (has) {
                 D = D_after;
                 R.T = T_after;
@@ -1668,7 +1765,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
         Replayer rp = {reg, min((int)uni_u32(reg[1]), P.rec_tile_words), 4, -1, false, RL};
         while (__any(R.active) && !rp.lost) {
             iteration([&](bool need, float, float, int &p0, bool &, float &found, float &searched_to, auto a, auto mid, auto b) {
-                return rp.slab(P, R, need, p0, found, searched_to, a, mid, b);
+                return rp.template slab<SUMS>(P, R, need, p0, found, searched_to, a, mid, b);
             });
         }
         replay_flush(P, RL);
@@ -1740,8 +1837,9 @@ __global__ __launch_bounds__(256) void k_tile_order(const MarchParams P)
 
 // The backward that searches the tree, and the one that replays the forward's record.  (Three
 // waves per SIMD with some spilling measured faster for the replay than two waves without.)
-__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchParams P) { march_bwd<false>(P); }
-__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay(const MarchParams P) { march_bwd<true>(P); }
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchParams P) { march_bwd<false, false>(P); }
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay(const MarchParams P) { march_bwd<true, false>(P); }
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay_sums(const MarchParams P) { march_bwd<true, true>(P); }
 
 // Test hook for the cooperative collect: per pixel a segment [tlo, thi] (thi < tlo = pixel idle);
 // writes each ray's hit count (negated when cut at cap) and the INPUT indices of its hits.
@@ -1900,6 +1998,9 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     const size_t order_words = (size_t)8 * g.per_xcd * g.bw * RGX_BLOCK_H;
     P.tile_order = M.order + order_words * sizeof(uint32_t) <= march_ws_bytes ? (uint32_t *)((char *)march_ws + M.order) : nullptr;
     P.use_tile_order = 0;
+    P.sum_pool = nullptr;
+    P.sum_next = nullptr;
+    P.sum_slots = 0;
     return RGX_OK;
 }
 
@@ -1919,7 +2020,17 @@ static int attach_records(MarchParams &P, void *records, size_t records_bytes)
     const size_t words = records_bytes / sizeof(uint32_t) / ntiles;
     if (((uintptr_t)records & 15u) || words < RGX_REC_MIN_TILE_WORDS) return RGX_EWORKSPACE;
     P.records = (uint32_t *)records;
-    P.rec_tile_words = (int32_t)(words > 0x3ffffff ? 0x3ffffff : words) & ~3;
+    if (words >= RGX_REC_LIST_WORDS + RGX_SUM_SLOT_WORDS) {
+        // room beyond the hit lists: RGX_REC_LIST_WORDS per tile, a 256-byte pool header, the sample-sum slots
+        P.rec_tile_words = RGX_REC_LIST_WORDS;
+        const size_t head = ntiles * (size_t)RGX_REC_LIST_WORDS * sizeof(uint32_t);
+        const size_t slots = (records_bytes - head - 256) / (RGX_SUM_SLOT_WORDS * sizeof(uint32_t));
+        P.sum_next = (uint32_t *)((char *)records + head);
+        P.sum_pool = (float4 *)((char *)records + head + 256);
+        P.sum_slots = (int32_t)(slots > 0x7fffffff ? 0x7fffffff : slots);
+    } else {
+        P.rec_tile_words = (int32_t)words & ~3;
+    }
     return RGX_OK;
 }
 
@@ -1941,8 +2052,12 @@ extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const Rgx
     if (rc) return rc;
     P.ray_colors = ray_colors;
     void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
-    if (P.records) hipLaunchKernelGGL((k_march_fwd<true, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
-    else hipLaunchKernelGGL((k_march_fwd<false, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    if (P.records) {
+        if (P.sum_pool) hipLaunchKernelGGL(k_zero4, dim3(1), dim3(64), 0, (hipStream_t)stream, (float4 *)P.sum_next, (int64_t)1);
+        hipLaunchKernelGGL((k_march_fwd<true, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    } else {
+        hipLaunchKernelGGL((k_march_fwd<false, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    }
     rgx_span_end(span, (hipStream_t)stream);
     RGX_LAUNCH_CHECK();
     return RGX_OK;
@@ -1987,6 +2102,7 @@ extern "C" int rgx_march_backward(const void *ws, const RgxCamera *cam, const Rg
             hipLaunchKernelGGL(k_tile_order, dim3(8), dim3(256), 0, s, P);
             P.use_tile_order = 1;
         }
+        if (P.sum_pool) hipLaunchKernelGGL(k_march_bwd_replay_sums, march_grid(P), dim3(64), 0, s, P);
         hipLaunchKernelGGL(k_march_bwd_replay, march_grid(P), dim3(64), 0, s, P);
         P.only_overflow = 1;
         P.use_tile_order = 0;

@@ -183,7 +183,10 @@ def _march_ws(n, n_rays, max_prim_slice, device):
     return _workspace("march", nbytes, device)
 
 
-REC_TILE_WORDS = 16384   # 64 KiB of hit-list record per 8x8 pixel tile
+# Record size per 8x8 pixel tile, 32-bit words: 16384 for the hit lists (64 KiB) and on average 64
+# slots of 8192 words for the per-sample density and colour sums of a slab iteration (the slots are
+# one pool shared by all tiles).  2.06 MiB per tile: 21 GB at 800x800.  16384 keeps the hit lists only.
+REC_TILE_WORDS = 16384 + 64 * 8192
 
 
 def new_records(cam, device, tile_words=REC_TILE_WORDS):

@@ -665,7 +665,7 @@ def test_direct_ctypes_binding_matches_the_python_mirror(gx, c0):
     s = C.c_void_p(torch.cuda.current_stream().cuda_stream)
     bvh = ws(lib.rgx_build_workspace_bytes, C.c_int64(N))
     mws = ws(lib.rgx_march_workspace_bytes, C.c_int64(N), C.c_int64(W * H), C.c_int32(cfg["max_prim_slice"]))
-    rec = ws(lib.rgx_march_records_bytes, C.c_int32(W), C.c_int32(H), C.c_int32(16384))
+    rec = ws(lib.rgx_march_records_bytes, C.c_int32(W), C.c_int32(H), C.c_int32(16384 + 64 * 8192))
     eye = (C.c_float * 3)(*camera.camera_center.tolist())
     f = dict(dtype=torch.float32, device=gx.DEV)
     rgb, prims, img = torch.empty(N, 3, **f), torch.empty(N, 16, **f), torch.empty(W * H, 3, **f)

@@ -311,8 +311,10 @@ __device__ __forceinline__ int delta(const uint64_t *keys, int64_t n, int64_t i,
     return 64 + __clz((int)((uint32_t)i ^ (uint32_t)j));
 }
 
+// other_end[i]: internal node i covers the sorted leaves between i and other_end[i]
 __global__ __launch_bounds__(256) void k_karras(const uint64_t *__restrict__ keys, int64_t n, Node *__restrict__ nodes,
-                                                int32_t *__restrict__ parent, int32_t *__restrict__ right)
+                                                int32_t *__restrict__ parent, int32_t *__restrict__ right,
+                                                int32_t *__restrict__ other_end)
 {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n - 1) return;
@@ -338,12 +340,17 @@ __global__ __launch_bounds__(256) void k_karras(const uint64_t *__restrict__ key
     right[i] = rc;
     parent[lc] = (int32_t)i;
     parent[rc] = (int32_t)i;
+    other_end[i] = (int32_t)j;
 }
 
 // Bottom-up refit: every leaf walks towards the root; the second thread to reach a node
-// (counted with an atomic) merges the two child boxes and goes on.  Box words travel between
-// threads through agent-scope atomic stores and loads (coherent across the XCDs' L2s without a
-// cache write-back); the workgroup-scope fences only order them against the counter.
+// (counted with an atomic) merges the two child boxes and goes on.  A workgroup owns 256
+// consecutive leaves of the sorted order; the nodes whose leaves all lie among them (internal node
+// i covers the leaves between i and other_end[i], so its index is one of them) are met in LDS:
+// counters, and the box of whichever child arrived first.  Only the few subtree roots a workgroup
+// ends up with go on through memory, where box words travel between threads through agent-scope
+// atomic stores and loads (coherent across the XCDs' L2s without a cache write-back); the
+// workgroup-scope fences only order them against the counter.
 __device__ __forceinline__ void st_agent(float *p, float v)
 {
     __hip_atomic_store((int *)p, __float_as_int(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -354,11 +361,45 @@ __device__ __forceinline__ float ld_agent(const float *p)
 }
 
 __global__ __launch_bounds__(256) void k_refit(int64_t n, Node *nodes, const int32_t *__restrict__ parent,
-                                               const int32_t *__restrict__ right, int32_t *flags)
+                                               const int32_t *__restrict__ right, const int32_t *__restrict__ other_end,
+                                               int32_t *flags)
 {
-    const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    __shared__ float s_box[2][6][256]; // [which child][lo xyz, hi xyz][node - first leaf of the workgroup]
+    __shared__ int s_arrived[256];
+    const int64_t b0 = (int64_t)blockIdx.x * 256, j = b0 + threadIdx.x;
+    s_arrived[threadIdx.x] = 0;
+    __syncthreads();
     if (j >= n) return;
-    int32_t node = parent[n - 1 + j];
+    const int64_t b1 = b0 + 255 < n - 1 ? b0 + 255 : n - 1;
+    int32_t child = (int32_t)(n - 1 + j);
+    float lo[3], hi[3];
+    for (int c = 0; c < 3; ++c) {
+        lo[c] = nodes[child].lo[c];
+        hi[c] = nodes[child].hi[c];
+    }
+    int32_t node = parent[child];
+    // nodes inside the workgroup's leaves: through LDS
+    while (node >= 0) {
+        const int32_t o = other_end[node];
+        if ((node < o ? node : o) < b0 || (node < o ? o : node) > b1) break;
+        const int slot = (int)(node - b0), side = nodes[node].left == child ? 0 : 1;
+        for (int c = 0; c < 3; ++c) {
+            s_box[side][c][slot] = lo[c];
+            s_box[side][3 + c][slot] = hi[c];
+        }
+        __threadfence_block();
+        if (atomicAdd(&s_arrived[slot], 1) == 0) return; // the sibling subtree is not done yet
+        __threadfence_block();
+        for (int c = 0; c < 3; ++c) {
+            lo[c] = fminf(lo[c], s_box[1 - side][c][slot]);
+            hi[c] = fmaxf(hi[c], s_box[1 - side][3 + c][slot]);
+            st_agent(&nodes[node].lo[c], lo[c]);
+            st_agent(&nodes[node].hi[c], hi[c]);
+        }
+        child = node;
+        node = parent[node];
+    }
+    // the rest of the way: through memory
     while (node >= 0) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (atomicAdd(&flags[node], 1) == 0) return; // the sibling subtree is not done yet
@@ -486,8 +527,9 @@ static int build_impl(const float *pos, const float *scale, const float *quat, c
         // 8 passes: the sorted keys / permutation are back in (k0, v0)
         hipLaunchKernelGGL(k_leaves, grid_for(n, 256), dim3(256), 0, s, boxes, v0, n, nodes, parent, flags);
         if (n > 1) {
-            hipLaunchKernelGGL(k_karras, grid_for(n - 1, 256), dim3(256), 0, s, k0, n, nodes, parent, right);
-            hipLaunchKernelGGL(k_refit, grid_for(n, 256), dim3(256), 0, s, n, nodes, parent, right, flags);
+            int32_t *other_end = (int32_t *)k1; // the sort's second key buffer is free again
+            hipLaunchKernelGGL(k_karras, grid_for(n - 1, 256), dim3(256), 0, s, k0, n, nodes, parent, right, other_end);
+            hipLaunchKernelGGL(k_refit, grid_for(n, 256), dim3(256), 0, s, n, nodes, parent, right, other_end, flags);
         }
         hipLaunchKernelGGL(k_skip_links, grid_for(2 * n - 1, 256), dim3(256), 0, s, n, nodes, parent, right);
     }

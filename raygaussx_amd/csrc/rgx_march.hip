@@ -14,10 +14,11 @@
 //      predicate for ITS ray and slab (so hit sets are those of a per-ray query); the result is,
 //      per 4x4 pixel row, the list of entries hit, and per lane its hit bits over that list;
 //   3. shades: every lane walks its own hits (forward, the backward's density pass), or the four
-//      rows walk their lists in lock step and sum each entry's 14 gradient words over the row's
-//      16 rays with DPP adds (the backward's gradient pass).
-// The forward can record what 1 and 2 produced; the replaying backward then needs no tree, no
-// table and no predicate, and sums a window's gradients in LDS before adding them to memory.
+//      rows walk their lists in lock step and sum each entry's 13 whitened-frame sums over the
+//      row's 16 rays with DPP adds (the backward's gradient pass).
+// The forward can record what 1 and 2 produced, and the per-sample density and colour sums of 3;
+// the replaying backward then needs no tree, no table, no predicate and no density pass, and
+// sums a window's gradients in LDS before adding them to memory.
 // The first-hit query (once per ray, and after an empty slab) runs on the same candidate tables.
 // The per-lane skip-link queries below serve the segment test hooks (arbitrary rays).
 #include "rgx_device.h"

@@ -655,11 +655,12 @@ __device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, f
 }
 
 // A Gaussian as the shading code sees it: its record in HBM plus its rotation columns,
-// inverse scales / k and k -- read from the LDS table entry when there is one, from the packed
-// 12-word frame (same operations, same values) that the replay keeps per window slot otherwise.
+// inverse scales / k and k -- read from the LDS table entry when there is one; otherwise the
+// rotation columns come from the 9-word frame the replay keeps per window slot (same operations,
+// same values) and the scales from the record.
 template <bool FROM_TABLE>
 struct Entry {
-    const float4 *tab; // LDS table entry (FROM_TABLE), or the replay's 3-word frame of the slot
+    const float4 *tab; // LDS table entry (FROM_TABLE), or the slot's column of the replay's frame array
     const Prim *prim;
     int32_t pid;       // index in Morton order
     int slot;          // its slot in the candidate table of the current window
@@ -671,10 +672,13 @@ struct Entry {
             inv = mk3(e3.x, e3.y, e3.z);
             k = e2.w;
         } else {
-            const float4 f0 = tab[0], f1 = tab[1], f2 = tab[2];
-            U = mk3(f0.x, f0.y, f0.z); V = mk3(f0.w, f1.x, f1.y); W = mk3(f1.z, f1.w, f2.x);
-            inv = mk3(f2.y, f2.z, f2.w);
-            k = prim->inv_inter4.w;
+            const float *f = (const float *)tab; // component-major: word c of this slot at f[c * RGX_CCAP]
+            U = mk3(f[0], f[RGX_CCAP], f[2 * RGX_CCAP]);
+            V = mk3(f[3 * RGX_CCAP], f[4 * RGX_CCAP], f[5 * RGX_CCAP]);
+            W = mk3(f[6 * RGX_CCAP], f[7 * RGX_CCAP], f[8 * RGX_CCAP]);
+            const float4 i4 = prim->inv_inter4;
+            inv = mk3(i4.x, i4.y, i4.z);
+            k = i4.w;
         }
     }
 };
@@ -1040,7 +1044,7 @@ __device__ __forceinline__ void sums_to_gradients(const Prim *pr, const float *s
 struct ReplayLds {
     float *acc;        // [RGX_NSUM][RGX_CCAP], component-major so that different slots fall in different banks
     uint32_t *pid;     // [RGX_CCAP]: the window's Gaussians by slot; top bit: the slot has something in acc
-    float4 *frame;     // [RGX_CCAP][3]: rotation columns U, V, W and (1/scale)/k of the window's Gaussians
+    float *frame;      // [9][RGX_CCAP]: rotation columns U, V, W of the window's Gaussians
 };
 
 __device__ __forceinline__ void replay_flush(const MarchParams &P, const ReplayLds &RL)
@@ -1076,12 +1080,12 @@ __device__ __forceinline__ void replay_window(const MarchParams &P, const Replay
         const uint32_t pid = min(reg[at + 4 + i], (uint32_t)(P.n - 1));
         RL.pid[i] = pid;
         const Prim *pr = P.prims + pid;
-        const float4 i4 = pr->inv_inter4;
         f3 U, V, W;
         quat_to_cols(pr->quat4, U, V, W);
-        RL.frame[3 * i] = make_float4(U.x, U.y, U.z, V.x);
-        RL.frame[3 * i + 1] = make_float4(V.y, V.z, W.x, W.y);
-        RL.frame[3 * i + 2] = make_float4(W.z, i4.x, i4.y, i4.z);
+        float *f = RL.frame + i;
+        f[0] = U.x; f[RGX_CCAP] = U.y; f[2 * RGX_CCAP] = U.z;
+        f[3 * RGX_CCAP] = V.x; f[4 * RGX_CCAP] = V.y; f[5 * RGX_CCAP] = V.z;
+        f[6 * RGX_CCAP] = W.x; f[7 * RGX_CCAP] = W.y; f[8 * RGX_CCAP] = W.z;
     }
     win_at = at;
     __syncthreads();
@@ -1123,7 +1127,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
                 bits &= bits - 1u;
             }
             const int32_t pid = (int32_t)(RL.pid[slot] & ~RGX_SLOT_TOUCHED);
-            body(Entry<false>{RL.frame + 3 * slot, P.prims + pid, pid, slot}, has, has, Half<(WALK & 1)>{});
+            body(Entry<false>{(const float4 *)(RL.frame + slot), P.prims + pid, pid, slot}, has, has, Half<(WALK & 1)>{});
         }
     } else {
         const int maxlen = min(max(max(l0, l1), max(l2, l3)), nw * 32);
@@ -1136,7 +1140,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
             if (__ballot(hit)) {
                 const int slot = live ? slots[i] & (RGX_CCAP - 1) : 0;
                 const int32_t pid = (int32_t)(RL.pid[slot] & ~RGX_SLOT_TOUCHED);
-                body(Entry<false>{RL.frame + 3 * slot, P.prims + pid, pid, slot}, hit, live, Half<0>{});
+                body(Entry<false>{(const float4 *)(RL.frame + slot), P.prims + pid, pid, slot}, hit, live, Half<0>{});
             }
         }
     }
@@ -1584,7 +1588,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
     const int lane = threadIdx.x;
     __shared__ float s_acc[REPLAY ? RGX_NSUM * RGX_CCAP : 1];
     __shared__ uint32_t s_pid[REPLAY ? RGX_CCAP : 1];
-    __shared__ float4 s_frame[REPLAY ? 3 * RGX_CCAP : 1];
+    __shared__ float s_frame[REPLAY ? 9 * RGX_CCAP : 1];
     const ReplayLds RL = {s_acc, s_pid, s_frame};
     if constexpr (REPLAY) {
         for (int i = lane; i < RGX_NSUM * RGX_CCAP; i += 64) s_acc[i] = 0.f;

@@ -746,7 +746,7 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
         }
         bits = first = second = 0;
     };
-    for (int h = 0; h < RGX_CCAP / 64; ++h) {
+    for (int h = 0; h < (RGX_CCAP + 63) / 64; ++h) {
         const int cl = h * 64 + lane;
         bool rel = false;
         if (cl < C) {
@@ -1123,7 +1123,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
             if (!__any(has)) break;
             int slot = 0;
             if (has) {
-                slot = slots[w * 32 + __builtin_ctz(bits)] & (RGX_CCAP - 1);
+                slot = min((int)slots[w * 32 + __builtin_ctz(bits)], RGX_CCAP - 1);
                 bits &= bits - 1u;
             }
             const int32_t pid = (int32_t)(RL.pid[slot] & ~RGX_SLOT_TOUCHED);
@@ -1138,7 +1138,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
             const bool hit = run && live && ((bits >> (i & 31)) & 1u);
             if (COUNT && hit) ++p0;
             if (__ballot(hit)) {
-                const int slot = live ? slots[i] & (RGX_CCAP - 1) : 0;
+                const int slot = live ? min((int)slots[i], RGX_CCAP - 1) : 0;
                 const int32_t pid = (int32_t)(RL.pid[slot] & ~RGX_SLOT_TOUCHED);
                 body(Entry<false>{(const float4 *)(RL.frame + slot), P.prims + pid, pid, slot}, hit, live, Half<0>{});
             }

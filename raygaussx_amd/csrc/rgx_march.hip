@@ -29,8 +29,9 @@
 #define RGX_QCAP 400       // node stack entries per wave (LDS)
 #endif
 #ifndef RGX_CCAP
-#define RGX_CCAP 128       // candidate table entries per wave (LDS)
+#define RGX_CCAP 112       // candidate table entries per wave (LDS): with 112 a tile needs 12 672 bytes, and 12 tiles fit a CU
 #endif
+#define RGX_MASK_WORDS ((RGX_CCAP + 31) / 32) // 32-bit words of a hit mask over a row's list
 #define RGX_DFS_MARGIN 128 // above QCAP - margin the sweep pops one node at a time (depth-first)
 #define RGX_LDS_HITS 32    // per-lane list of the stand-alone collect hook
 // The march kernels are sized (registers and LDS) for three wavefronts per SIMD.
@@ -355,7 +356,7 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
     const float4 *nodes4 = (const float4 *)P.nodes;
     const uint32_t n_nodes = (uint32_t)(2 * P.n - 1);
     int C = 0;
-    while ((S.qn > 0 || S.lqn > 0) && C + 64 <= RGX_CCAP) {
+    while ((S.qn > 0 || S.lqn > 0) && C < RGX_CCAP) {
         if (S.lqn >= 64 || S.qn == 0) {
             // Leaves whose boxes passed wait in a queue until there are 64 of them (or no node is
             // left): the expensive part -- fetch the Gaussian, test its ellipsoid, build its table
@@ -401,9 +402,16 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
                 }
                 leaf_hit = ok;
             }
+            // the table takes what it has room for; the rest goes back to the queue for the next table
+            const int rank = __popcll(__ballot(leaf_hit) & lt), room = RGX_CCAP - C;
+            const bool back = leaf_hit && rank >= room;
+            leaf_hit = leaf_hit && rank < room;
+            const uint64_t bb = __ballot(back);
+            if (back) s_leafq[S.lqn + __popcll(bb & lt)] = left;
+            S.lqn += __popcll(bb);
             const uint64_t bl = __ballot(leaf_hit);
             if (leaf_hit) {
-                float4 *dst = (float4 *)(s_tab + (C + __popcll(bl & lt)) * RGX_TAB);
+                float4 *dst = (float4 *)(s_tab + (C + rank) * RGX_TAB);
                 const f3 inv = mk3(p.inv_inter4.x, p.inv_inter4.y, p.inv_inter4.z);
                 const f3 O = mk3(p.pos4.x, p.pos4.y, p.pos4.z);
                 dst[0] = make_float4(U.x, U.y, U.z, dmin);
@@ -627,8 +635,8 @@ struct TileLds {
     int32_t *leafq;        // [128]: leaves waiting for the sweep's ellipsoid test
     float *tab;            // [RGX_CCAP * RGX_TAB]
     uint8_t *rowlist;      // [4][RGX_CCAP]: per 16-lane row, table slots some lane of the row hits
-    uint32_t (*mask)[64];  // [RGX_CCAP / 32][64]: per lane, hit bits over its row's list
-    uint32_t (*half)[4][RGX_CCAP / 32]; // [2][row][word]: list entries with samples in the slab's first / second 16
+    uint32_t (*mask)[64];  // [RGX_MASK_WORDS][64]: per lane, hit bits over its row's list
+    uint32_t (*half)[4][RGX_MASK_WORDS]; // [2][row][word]: list entries with samples in the slab's first / second 16
 };
 
 // Ray-interval-independent half of __intersection__gaussian (gaussians_aabb.cu:43-82) on a table
@@ -1391,8 +1399,8 @@ struct Replayer {
     __shared__ int32_t s_leafq[128];                                  \
     __shared__ __align__(16) float s_tab[RGX_CCAP * RGX_TAB];         \
     __shared__ uint8_t s_rowlist[4 * RGX_CCAP];                       \
-    __shared__ uint32_t s_mask[RGX_CCAP / 32][64];                    \
-    __shared__ uint32_t s_half[2][4][RGX_CCAP / 32];                  \
+    __shared__ uint32_t s_mask[RGX_MASK_WORDS][64];                   \
+    __shared__ uint32_t s_half[2][4][RGX_MASK_WORDS];                 \
     const TileLds L = {s_queue, s_leafq, s_tab, s_rowlist, s_mask, s_half}
 
 // lane -> pixel: row r = lane / 16 is the 4x4 block (r & 1, r >> 1) of the 8x8 tile

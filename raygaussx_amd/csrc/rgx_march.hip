@@ -26,10 +26,16 @@
 #include <type_traits>
 
 #ifndef RGX_QCAP
-#define RGX_QCAP 400       // node stack entries per wave (LDS)
+#define RGX_QCAP 432       // node stack entries per wave (LDS)
 #endif
 #ifndef RGX_CCAP
-#define RGX_CCAP 112       // candidate table entries per wave (LDS): with 112 a tile needs 12 672 bytes, and 12 tiles fit a CU
+#define RGX_CCAP 112       // candidate table entries per wave (LDS): with 112 (and a 432-entry stack) a tile needs 12 800 bytes, and 12 tiles fit a CU
+#endif
+#ifndef RGX_KHI
+#define RGX_KHI ((RGX_CCAP * 3) / 4) // a window that filled its table beyond this looks half as many slabs ahead next time
+#endif
+#ifndef RGX_KLO
+#define RGX_KLO (RGX_CCAP / 3)       // one that stayed below this, twice as many
 #endif
 #define RGX_MASK_WORDS ((RGX_CCAP + 31) / 32) // 32-bit words of a hit mask over a row's list
 #define RGX_DFS_MARGIN 128 // above QCAP - margin the sweep pops one node at a time (depth-first)
@@ -1234,8 +1240,8 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                         Wn.n = C;
                         Wn.resident = true;
                         Wn.crowded = false;
-                        if (C > (RGX_CCAP * 3) / 4) Wn.k = Wn.k > 1 ? Wn.k / 2 : 1;
-                        else if (C < RGX_CCAP / 3 && Wn.k < 32) Wn.k *= 2;
+                        if (C > RGX_KHI) Wn.k = Wn.k > 1 ? Wn.k / 2 : 1;
+                        else if (C < RGX_KLO && Wn.k < 32) Wn.k *= 2;
                     } else if (Wn.k > 1) {
                         Wn.k = 1; // too many Gaussians ahead: start over with this iteration's range only
                         frustum_range(F, t0, t1);

@@ -199,7 +199,7 @@ __global__ __launch_bounds__(256) void k_rs_scan_totals(uint32_t *__restrict__ t
     part[threadIdx.x] = v;
     __syncthreads();
     for (int o = 1; o < 256; o <<= 1) {
-        const uint32_t t = threadIdx.x >= o ? part[threadIdx.x - o] : 0u;
+        const uint32_t t = (int)threadIdx.x >= o ? part[threadIdx.x - o] : 0u;
         __syncthreads();
         part[threadIdx.x] += t;
         __syncthreads();

@@ -1869,7 +1869,7 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
     RGX_TILE_LDS();
     int px0, py0;
     if (!tile_origin(P, px0, py0)) return;
-    const int lane = threadIdx.x, row = lane >> 4;
+    const int lane = threadIdx.x;
     int px, py;
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;

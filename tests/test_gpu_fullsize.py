@@ -93,3 +93,25 @@ def test_renumbering_the_gaussians_permutes_the_gradients(gx, big):
     for k in PARAMS:
         cos, rel = gx.cos_rel(b["grads"][k], a["grads"][k][perm])
         assert cos >= 1 - 1e-6 and rel <= 1e-4, (k, cos, rel)
+
+
+def test_record_sizes_give_the_same_gradients(gx, big):
+    """The backward must not depend on how much of the forward's work the record kept: hit lists and
+    sample sums for every tile (the default), a pool of sample sums that runs out half way (tiles
+    with and without sums in one launch), hit lists only, and no record at all."""
+    sc, cam, cfg = big
+    g = np.random.default_rng(14).normal(size=(W * H, 3)).astype(np.float32)
+    _step("full size: default record")
+    ref = gx.gpu_render(sc, cam, cfg, want_grad=g)
+    assert ref["stats_bwd"]["nodes_visited"] == 0
+    for label, kw in (("sample-sum pool of 20 slots per tile", dict(rec_tile_words=16384 + 20 * 8192)),
+                      ("hit lists only", dict(rec_tile_words=16384)),
+                      ("no record", dict(record_hits=False))):
+        _step("full size: " + label)
+        out = gx.gpu_render(sc, cam, cfg, want_grad=g, **kw)
+        assert np.abs(out["image"] - ref["image"]).max() <= 2e-6
+        assert out["stats_bwd"]["hit_pairs"] == ref["stats_bwd"]["hit_pairs"]
+        assert (out["stats_bwd"]["nodes_visited"] > 0) == (label == "no record")
+        for k in PARAMS:
+            cos, rel = gx.cos_rel(out["grads"][k], ref["grads"][k])
+            assert cos >= 1 - 1e-6 and rel <= 1e-4, (label, k, cos, rel)

@@ -745,6 +745,8 @@ struct LaneQuery {
 // so that each half is shaded from its own, shorter list.  len (row-uniform) is the list length; p0 / ov count this lane's
 // hits and note the max_prim_slice cut (__anyhit__ah's optixTerminateRay, 352-356); found is
 // the running minimum of the searching lanes.
+// SEARCH: some lane of the wave is searching (otherwise the first-hit query's part is left out).
+template <bool SEARCH>
 __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, float t1, const LaneQuery &Q, int &p0, bool &ov,
                                              float &found, int &len, Counters &cn)
 {
@@ -776,11 +778,13 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
             float r1, r2;
             const bool ok = lane_roots((const float4 *)(L.tab + c * RGX_TAB), Q.dir, r1, r2);
             // first-hit query (searching lanes): smallest max(slo, r1) over the entries hit in [slo, shi]
-            const float ts = fmaxf(Q.slo, r1);
-            const bool sfound = Q.search && ok && ts <= fminf(Q.shi, r2);
-            found = sfound ? (found < 0.0f ? ts : fminf(found, ts)) : found;
+            if constexpr (SEARCH) {
+                const float ts = fmaxf(Q.slo, r1);
+                const bool sfound = Q.search && ok && ts <= fminf(Q.shi, r2);
+                found = sfound ? (found < 0.0f ? ts : fminf(found, ts)) : found;
+            }
             // collect query (marching lanes)
-            const bool seg = Q.need && !Q.search && !ov && ok && fmaxf(Q.tlo, r1) <= fminf(Q.thi, r2);
+            const bool seg = Q.need && !(SEARCH && Q.search) && !ov && ok && fmaxf(Q.tlo, r1) <= fminf(Q.thi, r2);
             const bool f = r1 < Q.tmid, g = r2 > Q.tmid;
             const bool counts = Q.part != 2 || !f;
             const bool over = seg && counts && p0 >= Q.cap;
@@ -1265,7 +1269,8 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                 int cnt = real ? p0 : q0;
                 bool cut = real ? ov : qov;
                 float best = phase == 0 ? found : -1.0f;
-                filter_table(L, C, lo, (phase == 0 && any_search) ? cover : hi, Q, cnt, cut, best, len, cn);
+                if (phase == 0 && any_search) filter_table<true>(L, C, lo, cover, Q, cnt, cut, best, len, cn);
+                else filter_table<false>(L, C, lo, hi, Q, cnt, cut, best, len, cn);
                 if (real) {
                     p0 = cnt;
                     ov = cut;

@@ -745,8 +745,9 @@ struct LaneQuery {
 // so that each half is shaded from its own, shorter list.  len (row-uniform) is the list length; p0 / ov count this lane's
 // hits and note the max_prim_slice cut (__anyhit__ah's optixTerminateRay, 352-356); found is
 // the running minimum of the searching lanes.
-// SEARCH: some lane of the wave is searching (otherwise the first-hit query's part is left out).
-template <bool SEARCH>
+// SEARCH: some lane of the wave is searching (otherwise the first-hit query's part is left out);
+// PART: LaneQuery::part, the same for all lanes.
+template <bool SEARCH, int PART>
 __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, float t1, const LaneQuery &Q, int &p0, bool &ov,
                                              float &found, int &len, Counters &cn)
 {
@@ -786,10 +787,10 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
             // collect query (marching lanes)
             const bool seg = Q.need && !(SEARCH && Q.search) && !ov && ok && fmaxf(Q.tlo, r1) <= fminf(Q.thi, r2);
             const bool f = r1 < Q.tmid, g = r2 > Q.tmid;
-            const bool counts = Q.part != 2 || !f;
+            const bool counts = PART != 2 || !f;
             const bool over = seg && counts && p0 >= Q.cap;
             ov = ov || over;
-            const bool hit = seg && !over && (Q.part == 0 || (Q.part == 1 ? f : g));
+            const bool hit = seg && !over && (PART == 0 || (PART == 1 ? f : g));
             p0 += (hit && counts) ? 1 : 0;
             const uint32_t in_first = (hit && f) ? 1u : 0u, in_second = (hit && g) ? 1u : 0u;
             const uint64_t bal = __ballot(hit);
@@ -1269,8 +1270,15 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                 int cnt = real ? p0 : q0;
                 bool cut = real ? ov : qov;
                 float best = phase == 0 ? found : -1.0f;
-                if (phase == 0 && any_search) filter_table<true>(L, C, lo, cover, Q, cnt, cut, best, len, cn);
-                else filter_table<false>(L, C, lo, hi, Q, cnt, cut, best, len, cn);
+                if (!split) {
+                    if (phase == 0 && any_search) filter_table<true, 0>(L, C, lo, cover, Q, cnt, cut, best, len, cn);
+                    else filter_table<false, 0>(L, C, lo, hi, Q, cnt, cut, best, len, cn);
+                } else if (phase == 0) {
+                    if (any_search) filter_table<true, 1>(L, C, lo, cover, Q, cnt, cut, best, len, cn);
+                    else filter_table<false, 1>(L, C, lo, hi, Q, cnt, cut, best, len, cn);
+                } else {
+                    filter_table<false, 2>(L, C, lo, hi, Q, cnt, cut, best, len, cn);
+                }
                 if (real) {
                     p0 = cnt;
                     ov = cut;

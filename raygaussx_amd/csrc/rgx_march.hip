@@ -469,23 +469,22 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
 }
 
 // Workgroups are dealt round-robin to the 8 XCDs (workgroup i runs on XCD i % 8), each with its
-// own L2.  The image is cut into blocks of RGX_BLOCK_W x RGX_BLOCK_H tiles and the blocks are
-// dealt to the XCDs in turn: an XCD works through adjacent tiles, so its L2 sees one region of
-// the scene at a time, and every XCD gets blocks from all over the image, so the expensive
-// middle of a scene is not one XCD's alone.  The number of blocks per row of blocks is kept odd
-// (by a phantom block column if need be): with an even count the same few block columns would go
-// to the same XCD in every row.
-#define RGX_BLOCK_W 4
-#define RGX_BLOCK_H 4
+// own L2.  The image is cut into square blocks of tiles and the blocks are dealt to the XCDs in
+// turn: an XCD works through adjacent tiles, so its L2 sees one region of the scene at a time, and
+// every XCD gets blocks from all over the image, so the expensive middle of a scene is not one
+// XCD's alone.  Blocks are 8 x 8 tiles where that still leaves every XCD some 32 blocks, else
+// 4 x 4.  The number of blocks per row of blocks is kept odd (by a phantom block column if need
+// be): with an even count the same few block columns would go to the same XCD in every row.
 struct TileGrid {
-    int bw, blocks_x, per_xcd; // block width in tiles (clipped to the image), blocks per row of blocks, blocks per XCD
+    int bw, bh, blocks_x, per_xcd; // block width (clipped to the image) and height in tiles, blocks per row of blocks, blocks per XCD
 };
 __host__ __device__ __forceinline__ TileGrid tile_grid(int tiles_x, int tiles_y)
 {
     TileGrid g;
-    g.bw = tiles_x < RGX_BLOCK_W ? tiles_x : RGX_BLOCK_W;
+    g.bh = ((tiles_x + 7) / 8) * ((tiles_y + 7) / 8) >= 256 ? 8 : 4;
+    g.bw = tiles_x < g.bh ? tiles_x : g.bh;
     g.blocks_x = ((tiles_x + g.bw - 1) / g.bw) | 1;
-    const int blocks_y = (tiles_y + RGX_BLOCK_H - 1) / RGX_BLOCK_H;
+    const int blocks_y = (tiles_y + g.bh - 1) / g.bh;
     g.per_xcd = (g.blocks_x * blocks_y + 7) >> 3;
     return g;
 }
@@ -493,13 +492,13 @@ __device__ __forceinline__ bool tile_origin(const MarchParams &P, int &px0, int 
 {
     const TileGrid g = tile_grid(P.tiles_x, P.tiles_y);
     const int xcd = blockIdx.x & 7;
-    const int per_block = g.bw * RGX_BLOCK_H;
+    const int per_block = g.bw * g.bh;
     int j = blockIdx.x >> 3;
     if (P.use_tile_order) j = (int)P.tile_order[xcd * (g.per_xcd * per_block) + j];
     int block = xcd + 8 * (j / per_block);
     const int within = j % per_block;
     const int tx = (block % g.blocks_x) * g.bw + within % g.bw;
-    const int ty = (block / g.blocks_x) * RGX_BLOCK_H + within / g.bw;
+    const int ty = (block / g.blocks_x) * g.bh + within / g.bw;
     px0 = tx * 8;
     py0 = ty * 8;
     if (tile_out) *tile_out = ty * P.tiles_x + tx;
@@ -1829,11 +1828,11 @@ __global__ __launch_bounds__(256) void k_tile_order(const MarchParams P)
     __shared__ uint32_t s_bin[RGX_ORDER_BINS];
     __shared__ uint32_t s_part[256];
     const TileGrid g = tile_grid(P.tiles_x, P.tiles_y);
-    const int per_block = g.bw * RGX_BLOCK_H, cnt = g.per_xcd * per_block, xcd = blockIdx.x;
+    const int per_block = g.bw * g.bh, cnt = g.per_xcd * per_block, xcd = blockIdx.x;
     auto size_class = [&](int j) -> uint32_t {
         const int block = xcd + 8 * (j / per_block), within = j % per_block;
         const int tx = (block % g.blocks_x) * g.bw + within % g.bw;
-        const int ty = (block / g.blocks_x) * RGX_BLOCK_H + within / g.bw;
+        const int ty = (block / g.blocks_x) * g.bh + within / g.bw;
         if (tx >= P.tiles_x || ty >= P.tiles_y) return 0u;
         const uint32_t *reg = P.records + (int64_t)(ty * P.tiles_x + tx) * P.rec_tile_words;
         if (!record_usable(P, reg)) return 0u;
@@ -2027,7 +2026,7 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     P.only_overflow = 0;
     // room for the tile order?  (a workspace sized for fewer rays, or an image of extreme proportions, goes without)
     const TileGrid g = tile_grid(P.tiles_x, P.tiles_y);
-    const size_t order_words = (size_t)8 * g.per_xcd * g.bw * RGX_BLOCK_H;
+    const size_t order_words = (size_t)8 * g.per_xcd * g.bw * g.bh;
     P.tile_order = M.order + order_words * sizeof(uint32_t) <= march_ws_bytes ? (uint32_t *)((char *)march_ws + M.order) : nullptr;
     P.use_tile_order = 0;
     P.sum_pool = nullptr;
@@ -2069,7 +2068,7 @@ static int attach_records(MarchParams &P, void *records, size_t records_bytes)
 static inline dim3 march_grid(const MarchParams &P)
 {
     const TileGrid g = tile_grid(P.tiles_x, P.tiles_y);
-    return dim3((unsigned)(8 * g.per_xcd * g.bw * RGX_BLOCK_H));
+    return dim3((unsigned)(8 * g.per_xcd * g.bw * g.bh));
 }
 
 extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,

@@ -731,8 +731,6 @@ struct LaneQuery {
     float slo, shi;
     int cap;        // max_prim_slice
     float tmid;     // tbuffer + 16 dt: where the slab's second 16 samples begin
-    int part;       // 0: all hits of [tlo, thi]; 1: only those reaching the first 16 samples; 2: only those
-                    // reaching the second 16, of which the ones that also reach the first are not counted again
 };
 
 // Filter: every lane tests the table entries whose distance shell meets [t0, t1] (the union of
@@ -744,8 +742,10 @@ struct LaneQuery {
 // so that each half is shaded from its own, shorter list.  len (row-uniform) is the list length; p0 / ov count this lane's
 // hits and note the max_prim_slice cut (__anyhit__ah's optixTerminateRay, 352-356); found is
 // the running minimum of the searching lanes.
-// SEARCH: some lane of the wave is searching (otherwise the first-hit query's part is left out);
-// PART: LaneQuery::part, the same for all lanes.
+// SEARCH: some lane of the wave is searching (otherwise the first-hit query's part is left out).
+// PART (the same for all lanes): 0: all hits of [tlo, thi]; 1: only those reaching the first 16
+// samples; 2: only those reaching the second 16, of which the ones that also reach the first are
+// not counted again.
 template <bool SEARCH, int PART>
 __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, float t1, const LaneQuery &Q, int &p0, bool &ov,
                                              float &found, int &len, Counters &cn)
@@ -1263,8 +1263,7 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
             if (phase == 0 || !Wn.resident || split) {
                 // phase 0 asks the lane's real question; a phase-1 re-filter only recounts the slab hits
                 const float cover = split ? hi : (Wn.resident ? Wn.hi : t1); // this iteration's tables cover [t0, cover]
-                const LaneQuery Q = {R.dir, run, tlo, thi, phase == 0 && srch, R.tbuffer, fminf(R.texit, cover), P.m.max_prim_slice,
-                                     tmid, split ? phase + 1 : 0};
+                const LaneQuery Q = {R.dir, run, tlo, thi, phase == 0 && srch, R.tbuffer, fminf(R.texit, cover), P.m.max_prim_slice, tmid};
                 const bool real = phase == 0 || split; // counts into the lane's own p0 / ov
                 int cnt = real ? p0 : q0;
                 bool cut = real ? ov : qov;

@@ -1474,7 +1474,6 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
 #pragma unroll
             for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
             f3 rdt = dir * fmaf(dt, 0.5f, R.tbuffer); // samples 0..15
-            float t_sample = R.tbuffer + 0.5f * dt;
             auto accumulate = [&](const auto &e, bool hit, bool, auto) {
                 if (hit) {
                     const float4 col = e.prim->rgba4;
@@ -1495,7 +1494,14 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
                     }
                 }
             };
-            auto blend = [&]() { // gaussians_aabb.cu:195-201
+            auto blend = [&](bool second_chunk) { // gaussians_aabb.cu:195-201
+                float t_sample = R.tbuffer + 0.5f * dt; // the viewer's running sample position (cuda_gui/gaussians_aabb.cu:189)
+                if constexpr (VIEWER) {
+                    if (second_chunk) {
+#pragma unroll
+                        for (int i = 0; i < RGX_CHUNK_SIZE; ++i) t_sample += dt; // as the first chunk left it
+                    }
+                }
 #pragma unroll
                 for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
                     const float x = sg[i] * dt;
@@ -1532,7 +1538,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
             };
             auto second_half = [&](bool split) { // split: the hits of the second half are not known yet
                 const bool has = need && (p0 > 0 || split);
-                if (has) blend();
+                if (has) blend(false);
                 keep_sums(0);
                 // samples 16..31, only for rays still above the transmittance floor (gaussians_aabb.cu:190)
 #pragma unroll
@@ -1542,7 +1548,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
             };
             const bool run2 = slab_tables<WALK_FORWARD>(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, accumulate,
                                           second_half, accumulate);
-            if (run2) blend();
+            if (run2) blend(true);
             keep_sums(RGX_CHUNK_SIZE);
             if (need && p0 > 0) {
                 cn.slabs++;

@@ -115,3 +115,32 @@ def test_record_sizes_give_the_same_gradients(gx, big):
         for k in PARAMS:
             cos, rel = gx.cos_rel(out["grads"][k], ref["grads"][k])
             assert cos >= 1 - 1e-6 and rel <= 1e-4, (label, k, cos, rel)
+
+
+def test_large_image_of_a_small_scene(gx, orc):
+    """Images beyond about a megapixel are dealt to the XCDs in 8x8-tile blocks instead of 4x4 (a
+    ragged 1101x1003 image here: 138x126 tiles, the last column and row partly outside).  Colours and
+    gradients of a ray sample spread over the whole image against the oracle; an unmapped or
+    doubly mapped block of tiles would show in both."""
+    w, h = 1101, 1003
+    sc = scenes.scene_to_numpy(scenes.make_scene(1, n=20000, seed=5))
+    sc = {k: sc[k] for k in PARAMS}
+    sc["scales"] = sc["scales"] * 3.0
+    cam, cfg = scenes.make_camera(1, 2, width=w, height=h), scenes.CONFIGS[1]
+    ids = np.unique(np.random.default_rng(15).integers(0, w * h, 3000))
+    img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"], ray_ids=ids)
+    dloss = np.zeros((w * h, 3), np.float32)
+    dloss[ids] = np.random.default_rng(16).normal(size=(len(ids), 3)).astype(np.float32)
+    og, ost = orc.render_backward(sc, ctx, img, dloss)
+    _step("1101x1003 image, 20000 Gaussians")
+    out = gx.gpu_render(sc, cam, cfg, want_grad=dloss)
+    assert st["hit_pairs"] > 20000
+    assert np.abs(out["image"][ids] - img[ids]).max() <= IMG_TOL
+    # every pixel was written: colours in range, none left at the all-zero of fresh memory, background white
+    assert 0.0 <= out["image"].min() and out["image"].max() <= 1.0 + 1e-5
+    assert not np.any(np.all(out["image"] == 0.0, axis=1))
+    assert np.all(out["image"] == 1.0, axis=1).mean() > 0.2
+    assert out["stats_fwd"]["hit_pairs"] == out["stats_bwd"]["hit_pairs"]
+    for k in PARAMS:
+        cos, rel = gx.cos_rel(out["grads"][k], og[k])
+        assert cos >= COS_MIN and rel <= REL_MAX, (k, cos, rel)

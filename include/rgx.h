@@ -231,6 +231,15 @@ int rgx_collect_tiles(const void *ws, const RgxCamera *cam, const float *prims, 
                       const float *tlo, const float *thi, int32_t cap, int32_t *counts, int32_t *ids,
                       void *stream);
 
+/* Test hook for the arithmetic of the hit predicate.  Where a Gaussian's scales and distance are of
+ * ordinary size the kernels form the predicate's two quotients and its square root
+ * (gaussians_aabb.cu:59-75) with the compiler's own instruction sequences for `/` and sqrtf()
+ * minus their handling of extreme exponents.  This counts, over n pairs (a[i], b[i]) of device
+ * floats, those for which a / b, 1 / b, sqrt(|a|) or sqrt(2^-40 |a|) so formed differ in any bit
+ * from the full sequences; *bad (device, cleared by the caller) receives the count, 0 for operands in range
+ * (2^-46 <= |a|, |b| <= 2^46). */
+int rgx_check_plain_arith(const float *a, const float *b, int64_t n, uint32_t *bad, void *stream);
+
 /* ---- Morton reordering of the point cloud --------------------------------- */
 
 /* Replaces quantify_pos_min_max + morton_code + argsort (utils/reordering_utils.py:55-104,

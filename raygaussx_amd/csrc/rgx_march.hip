@@ -286,6 +286,38 @@ __device__ __forceinline__ bool frustum_overlaps(const Frustum &F, float4 a, flo
 // if it still passes, written to the candidate table.  Returns the number of table entries
 // when the stack is empty (done) or the table might not take another step's leaves; call again
 // to continue with an emptied table.
+// Correctly rounded a / b and sqrt(x) for operands of ordinary size: the instruction sequences the
+// compiler emits for `/` and sqrtf(), without their range handling (v_div_scale / v_div_fixup,
+// the 2^32 pre-scaling of small sqrt arguments, the special-value checks).  Where that handling
+// would do nothing -- b and a / b far from the ends of the exponent range, |a| >= 2^-104,
+// 2^-96 <= x < infinity -- the results are bit-identical to `/` and sqrtf().
+__device__ __forceinline__ float div_rn_plain(float a, float b)
+{
+    float r = __builtin_amdgcn_rcpf(b);
+    r = fmaf(fmaf(-b, r, 1.0f), r, r);
+    float q = a * r;
+    q = fmaf(fmaf(-b, q, a), r, q);
+    return fmaf(fmaf(-b, q, a), r, q);
+}
+__device__ __forceinline__ float sqrt_rn_plain(float x)
+{
+    const float y = __builtin_amdgcn_sqrtf(x); // within one ulp: the answer is y or a neighbour
+    const float down = __int_as_float(__float_as_int(y) - 1), up = __int_as_float(__float_as_int(y) + 1);
+    const float r_down = fmaf(-down, y, x), r_up = fmaf(-up, y, x);
+    const float z = r_down <= 0.0f ? down : y;
+    return r_up > 0.0f ? up : z;
+}
+
+// Whether the divisions and the square root of lane_roots() may take the plain forms for every
+// ray through a Gaussian: inv = (1 / scale) / k per axis, c = |S^-1 R^T (eye - centre)|^2 - 1.
+// For a unit direction a = |De|^2 lies in [min inv^2, max inv^2]; where the line hits
+// (disc > 1e-7) disc * a >= 1e-7 min inv^2 and |q| lies in [sqrt(1e-7) min inv, (sqrt(c + 1) + 1) max inv].
+__device__ __forceinline__ bool plain_roots(f3 inv, float c)
+{
+    const float lo = fminf(inv.x, fminf(inv.y, inv.z)), hi = fmaxf(inv.x, fmaxf(inv.y, inv.z));
+    return lo >= 0x1p-23f && hi <= 0x1p22f && fabsf(c) >= 0x1p-46f && fabsf(c) <= 0x1p46f;
+}
+
 struct Sweep {
     int qn;  // stack entries (wave-uniform)
     int lqn; // leaves waiting for their ellipsoid test (wave-uniform)
@@ -354,9 +386,12 @@ __device__ __forceinline__ void frustum_cut(const MarchParams &P, Frustum &F, fl
     if (have != (count >= 64 ? ~0ull : ((1ull << count) - 1ull))) F.cut_n = 0; // (cannot happen) fall back to the root
 }
 
+// Fills the table from the sweep; returns the number of entries.  done: the sweep is finished;
+// plain: every entry passed plain_roots().
 __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int32_t *s_queue, int32_t *s_leafq, float *s_tab,
-                          bool &done, Counters &cn)
+                          bool &done, bool &plain, Counters &cn)
 {
+    plain = true;
     const int lane = threadIdx.x;
     const uint64_t lt = (1ull << lane) - 1ull;
     const float4 *nodes4 = (const float4 *)P.nodes;
@@ -424,9 +459,12 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
                 dst[1] = make_float4(V.x, V.y, V.z, dmax);
                 dst[2] = make_float4(W.x, W.y, W.z, p.inv_inter4.w);
                 const f3 Oe = apply_sinv_rt(O, U, V, W, inv);
-                dst[3] = make_float4(inv.x, inv.y, inv.z, fmaf(Oe.x, Oe.x, fmaf(Oe.y, Oe.y, fmaf(Oe.z, Oe.z, -1.0f))));
+                const float c = fmaf(Oe.x, Oe.x, fmaf(Oe.y, Oe.y, fmaf(Oe.z, Oe.z, -1.0f)));
+                dst[3] = make_float4(inv.x, inv.y, inv.z, c);
                 dst[4] = make_float4(Oe.x, Oe.y, Oe.z, __int_as_float(~left));
+                leaf_hit = plain_roots(inv, c); // from here on: this lane's entry is a plain one
             }
+            plain = plain && __ballot(leaf_hit) == bl;
             C += __popcll(bl);
             __syncthreads();
             continue;
@@ -645,7 +683,9 @@ struct TileLds {
 };
 
 // Ray-interval-independent half of __intersection__gaussian (gaussians_aabb.cu:43-82) on a table
-// entry: same arithmetic as line_roots(), with the precomputed ray-independent parts.
+// entry: same arithmetic as line_roots(), with the precomputed ray-independent parts.  PLAIN: the
+// entry passed plain_roots().
+template <bool PLAIN>
 __device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, float &r2)
 {
     const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3], e4 = e[4];
@@ -654,15 +694,15 @@ __device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, f
     const float a = fmaf(De.x, De.x, fmaf(De.y, De.y, De.z * De.z));
     const float b = -fmaf(Oe.x, De.x, fmaf(Oe.y, De.y, Oe.z * De.z));
     const float c = e3.w;
-    const float inv_a = 1.0f / a;
+    const float inv_a = PLAIN ? div_rn_plain(1.0f, a) : 1.0f / a;
     const float b_inv_a = b * inv_a;
     const f3 Pc = mk3(fmaf(b_inv_a, De.x, Oe.x), fmaf(b_inv_a, De.y, Oe.y), fmaf(b_inv_a, De.z, Oe.z));
     const float d2 = fmaf(Pc.x, Pc.x, fmaf(Pc.y, Pc.y, Pc.z * Pc.z));
     const float disc = 1.0f - d2;
     // no branch: where the line misses (disc <= 1e-7) the roots are garbage and the result false
-    const float sdisc = sqrtf(disc * a);
+    const float sdisc = PLAIN ? sqrt_rn_plain(disc * a) : sqrtf(disc * a);
     const float q = b + copysignf(sdisc, b);
-    r1 = c / q;
+    r1 = PLAIN ? div_rn_plain(c, q) : c / q;
     r2 = q * inv_a;
     return disc > 1e-7f;
 }
@@ -745,8 +785,8 @@ struct LaneQuery {
 // SEARCH: some lane of the wave is searching (otherwise the first-hit query's part is left out).
 // PART (the same for all lanes): 0: all hits of [tlo, thi]; 1: only those reaching the first 16
 // samples; 2: only those reaching the second 16, of which the ones that also reach the first are
-// not counted again.
-template <bool SEARCH, int PART>
+// not counted again.  PLAIN: every entry of the table passed plain_roots().
+template <bool SEARCH, int PART, bool PLAIN>
 __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, float t1, const LaneQuery &Q, int &p0, bool &ov,
                                              float &found, int &len, Counters &cn)
 {
@@ -776,7 +816,7 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
             m &= m - 1;
             // straight-line code: every lane evaluates both queries' predicates, its state selects
             float r1, r2;
-            const bool ok = lane_roots((const float4 *)(L.tab + c * RGX_TAB), Q.dir, r1, r2);
+            const bool ok = lane_roots<PLAIN>((const float4 *)(L.tab + c * RGX_TAB), Q.dir, r1, r2);
             // first-hit query (searching lanes): smallest max(slo, r1) over the entries hit in [slo, shi]
             if constexpr (SEARCH) {
                 const float ts = fmaxf(Q.slo, r1);
@@ -1173,6 +1213,7 @@ struct Window {
     bool resident;
     int k;        // slabs to look ahead when a window is built
     bool crowded; // the last iteration's Gaussians did not fit one table
+    bool plain;   // the resident table's entries all passed plain_roots()
 };
 
 __device__ __forceinline__ void frustum_range(Frustum &F, float t0, float t1)
@@ -1230,12 +1271,14 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
         bool first = true, more = true;
         while (more) {
             int C;
+            bool plain;
             if (reuse) {
                 C = Wn.n;
+                plain = Wn.plain;
                 more = false;
             } else {
                 bool done;
-                C = sweep_next(P, S, F, L.queue, L.leafq, L.tab, done, cn);
+                C = sweep_next(P, S, F, L.queue, L.leafq, L.tab, done, plain, cn);
                 if (split) {
                     seen += C;
                 } else if (phase == 0 && first) {
@@ -1243,6 +1286,7 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                         Wn.hi = F.t1;
                         Wn.n = C;
                         Wn.resident = true;
+                        Wn.plain = plain;
                         Wn.crowded = false;
                         if (C > RGX_KHI) Wn.k = Wn.k > 1 ? Wn.k / 2 : 1;
                         else if (C < RGX_KLO && Wn.k < 32) Wn.k *= 2;
@@ -1268,14 +1312,20 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                 int cnt = real ? p0 : q0;
                 bool cut = real ? ov : qov;
                 float best = phase == 0 ? found : -1.0f;
+                auto filter = [&](auto search, auto part) {
+                    const float far = decltype(search)::value ? cover : hi;
+                    if (std::is_same<Rec, NoRecorder>::value ? __builtin_expect(plain, 1) : plain) filter_table<decltype(search)::value, decltype(part)::value, true>(L, C, lo, far, Q, cnt, cut, best, len, cn);
+                    else filter_table<decltype(search)::value, decltype(part)::value, false>(L, C, lo, far, Q, cnt, cut, best, len, cn);
+                };
+                using std::integral_constant;
                 if (!split) {
-                    if (phase == 0 && any_search) filter_table<true, 0>(L, C, lo, cover, Q, cnt, cut, best, len, cn);
-                    else filter_table<false, 0>(L, C, lo, hi, Q, cnt, cut, best, len, cn);
+                    if (phase == 0 && any_search) filter(std::true_type{}, integral_constant<int, 0>{});
+                    else filter(std::false_type{}, integral_constant<int, 0>{});
                 } else if (phase == 0) {
-                    if (any_search) filter_table<true, 1>(L, C, lo, cover, Q, cnt, cut, best, len, cn);
-                    else filter_table<false, 1>(L, C, lo, hi, Q, cnt, cut, best, len, cn);
+                    if (any_search) filter(std::true_type{}, integral_constant<int, 1>{});
+                    else filter(std::false_type{}, integral_constant<int, 1>{});
                 } else {
-                    filter_table<false, 2>(L, C, lo, hi, Q, cnt, cut, best, len, cn);
+                    filter(std::false_type{}, integral_constant<int, 2>{});
                 }
                 if (real) {
                     p0 = cnt;
@@ -1460,7 +1510,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
     frustum_cut(P, F, wave_max_all(R.active && R.texit < 1e30f ? R.texit : 0.f), L.queue);
     const f3 dir = R.dir;
     float Cr = 0.f, Cg = 0.f, Cb = 0.f, depth = 0.f;
-    Window Wn = {0.f, 0, false, 4, false};
+    Window Wn = {0.f, 0, false, 4, false, false};
 
     while (__any(R.active)) {
         float tlo, thi;
@@ -1811,7 +1861,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
         Frustum F;
         frustum_planes(P.cam, px0, py0, F);
         frustum_cut(P, F, wave_max_all(R.active && R.texit < 1e30f ? R.texit : 0.f), L.queue);
-        Window Wn = {0.f, 0, false, 4, false};
+        Window Wn = {0.f, 0, false, 4, false, false};
         NoRecorder rec;
         while (__any(R.active)) {
             iteration([&](bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to, auto a, auto mid,
@@ -1908,7 +1958,7 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
         R.tbuffer = tlo;
         R.texit = thi;
         R.slab_spacing = 0.f;
-        Window Wn = {0.f, 0, false, 1, false};
+        Window Wn = {0.f, 0, false, 1, false, false};
         float found = -1.0f, searched_to = 0.f;
         MarchParams Pc = P;
         Pc.m.max_prim_slice = cap;
@@ -2208,6 +2258,29 @@ extern "C" int rgx_collect_tiles(const void *ws, const RgxCamera *cam, const flo
     P.tiles_x = (cam->width + 7) / 8;
     P.tiles_y = (cam->height + 7) / 8;
     hipLaunchKernelGGL(k_collect_tiles, march_grid(P), dim3(64), 0, (hipStream_t)stream, P, tlo, thi, (int)cap, counts, ids);
+    RGX_LAUNCH_CHECK();
+    return RGX_OK;
+}
+
+// Test hook: counts the pairs for which the plain division or the plain square root differs in any
+// bit from `/` or sqrtf() (expected: none, for operands inside the ranges plain_roots() grants).
+__global__ __launch_bounds__(256) void k_check_plain_arith(const float *__restrict__ a, const float *__restrict__ b, int64_t n,
+                                                           uint32_t *bad)
+{
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float x = a[i], y = b[i];
+    const bool same = __float_as_uint(div_rn_plain(x, y)) == __float_as_uint(x / y) &&
+                      __float_as_uint(div_rn_plain(1.0f, y)) == __float_as_uint(1.0f / y) &&
+                      __float_as_uint(sqrt_rn_plain(fabsf(x))) == __float_as_uint(sqrtf(fabsf(x))) &&
+                      __float_as_uint(sqrt_rn_plain(fabsf(x) * 0x1p-40f)) == __float_as_uint(sqrtf(fabsf(x) * 0x1p-40f));
+    if (!same) atomicAdd(bad, 1u);
+}
+
+extern "C" int rgx_check_plain_arith(const float *a, const float *b, int64_t n, uint32_t *bad, void *stream)
+{
+    if (n < 0 || (n > 0 && (!a || !b)) || !bad) return RGX_EINVAL;
+    if (n > 0) hipLaunchKernelGGL(k_check_plain_arith, grid_for(n, 256), dim3(256), 0, (hipStream_t)stream, a, b, n, bad);
     RGX_LAUNCH_CHECK();
     return RGX_OK;
 }

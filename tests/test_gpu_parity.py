@@ -726,3 +726,39 @@ def test_empty_cloud_and_one_pixel_image(gx):
     assert out["image"].shape == (1, 3) and np.isfinite(out["image"]).all()
     assert out["stats_fwd"]["hit_pairs"] == out["stats_bwd"]["hit_pairs"] > 0
     assert np.isfinite(out["grads"]["positions"]).all() and np.abs(out["grads"]["positions"]).sum() > 0
+
+
+def test_plain_division_and_square_root_are_correctly_rounded(gx):
+    """The hit predicate's quotients and square root are formed without the compiler's handling of
+    extreme exponents wherever a Gaussian's scales and distance allow (which is everywhere in
+    practice).  Inside the granted range the short forms must equal `/` and sqrtf() in every bit:
+    8 million operand pairs with exponents over the whole range and mantissas that include the
+    all-zeros / all-ones patterns and near-ties."""
+    import ctypes as C
+    from raygaussx_amd import _lib
+    rng = np.random.default_rng(31)
+    n = 1 << 23
+
+    def operands():
+        mant = rng.integers(0, 1 << 23, n, dtype=np.uint32)
+        special = rng.integers(0, 8, n)
+        mant = np.where(special == 0, 0, mant)
+        mant = np.where(special == 1, (1 << 23) - 1, mant)
+        mant = np.where(special == 2, mant & 0x7, mant)              # just above a power of two
+        mant = np.where(special == 3, mant | 0x7FFFF8, mant)         # just below one
+        expo = rng.integers(127 - 46, 127 + 46, n, dtype=np.uint32)  # 2^-46 <= |v| < 2^46
+        sign = rng.integers(0, 2, n, dtype=np.uint32)
+        return ((sign << 31) | (expo << 23) | mant.astype(np.uint32)).astype(np.uint32).view(np.float32)
+
+    a, b = torch.from_numpy(operands()).to(gx.DEV), torch.from_numpy(operands()).to(gx.DEV)
+    bad = torch.zeros(1, dtype=torch.int32, device=gx.DEV)
+    _step("plain division / square root against the full sequences")
+    _lib.check(_lib.lib().rgx_check_plain_arith(_lib.ptr(a), _lib.ptr(b), C.c_int64(n), _lib.ptr(bad), _lib.stream()))
+    torch.cuda.synchronize()
+    assert int(bad.item()) == 0
+    # and the check itself can fail: far outside the range the short division loses its footing
+    tiny = torch.full((1024,), 1e-38, dtype=torch.float32, device=gx.DEV)
+    huge = torch.full((1024,), 3e38, dtype=torch.float32, device=gx.DEV)
+    _lib.check(_lib.lib().rgx_check_plain_arith(_lib.ptr(tiny), _lib.ptr(huge), C.c_int64(1024), _lib.ptr(bad), _lib.stream()))
+    torch.cuda.synchronize()
+    assert int(bad.item()) > 0

@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 import torch
 
-from raygaussx_amd import _lib, scenes
+from raygaussx_amd import _lib, scenes, optix_utils as u_ox
 
 HEADER = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "include", "rgx.h")
 
@@ -45,11 +45,18 @@ def test_error_strings_and_size_queries():
     assert lib.rgx_build_workspace_bytes(C.c_int64(-1), C.byref(out)) == -1
     assert lib.rgx_build_workspace_bytes(C.c_int64(5), None) == -1
     assert lib.rgx_march_workspace_bytes(C.c_int64(1000), C.c_int64(640000), C.c_int32(2048), C.byref(out)) == 0
-    assert out.value >= 1000 * 64
+    with_rays = out.value
+    assert lib.rgx_march_workspace_bytes(C.c_int64(1000), C.c_int64(0), C.c_int32(2048), C.byref(out)) == 0
+    # the gradient block (64 bytes per Gaussian) and, growing with the ray count, the tile order of the backward
+    assert 1000 * 64 <= out.value < with_rays and with_rays % 256 == 0 and with_rays - out.value >= (640000 // 64) * 4
     assert lib.rgx_march_records_bytes(C.c_int32(800), C.c_int32(800), C.c_int32(16384), C.byref(out)) == 0
     assert out.value == 100 * 100 * 16384 * 4
     assert lib.rgx_march_records_bytes(C.c_int32(801), C.c_int32(9), C.c_int32(1024), C.byref(out)) == 0
     assert out.value == 101 * 2 * 1024 * 4
+    # hit lists plus on average 64 slots of sample sums per tile (the Python mirror's default)
+    assert lib.rgx_march_records_bytes(C.c_int32(800), C.c_int32(800), C.c_int32(u_ox.REC_TILE_WORDS), C.byref(out)) == 0
+    assert u_ox.REC_TILE_WORDS == 16384 + 64 * 8192 and out.value == 100 * 100 * u_ox.REC_TILE_WORDS * 4
+    assert lib.rgx_check_plain_arith(None, None, C.c_int64(4), None, None) == -1
     for bad in ((0, 8, 16384), (8, 8, 512), (8, 8, 1026)):     # empty image, region too small, not a multiple of 4
         assert lib.rgx_march_records_bytes(C.c_int32(bad[0]), C.c_int32(bad[1]), C.c_int32(bad[2]), C.byref(out)) == -1
     assert lib.rgx_morton_workspace_bytes(C.c_int64(1000), C.byref(out)) == 0 and out.value > 0

@@ -80,6 +80,12 @@ def set_num_threads(n):
     lib().orc_set_num_threads(int(n))
 
 
+def set_step_scale(scale):
+    """Scale the adaptive step's coefficient 1 / cbrt(T) (1.0: the reference's arithmetic).  A probe
+    for how far a last-bit difference in cbrt moves the results of ``dynamic_sampling``."""
+    lib().orc_set_step_scale(C.c_float(scale))
+
+
 def camera_struct(cam, supersampling=(1, 1)):
     """``cam`` exposes the reference Camera attributes read at optix_utils.py:258-266."""
     c = OrcCamera()

@@ -88,6 +88,7 @@ static inline float dot3(f3 a, f3 b) { return (a.x * b.x + a.y * b.y) + a.z * b.
 /* vec_math.h:554-558 normalize: v * (1/sqrtf(dot(v,v))) */
 static inline f3 normalize3(f3 v) { float inv = 1.0f / sqrtf(dot3(v, v)); return scl3(v, inv); }
 static inline float canon_logf(float x) { return (float)log((double)x); }
+static float g_step_scale = 1.0f; /* see orc_set_step_scale() */
 
 /* cuda_train/forward/gaussians_aabb.cu:7-17 quaternion_to_matrix (columns of R) */
 static inline void quat_to_cols(const float *q, f3 *c0, f3 *c1, f3 *c2)
@@ -543,7 +544,7 @@ static void march_forward_ray(const OrcCamera *cam, const OrcMarch *m, const flo
     while (tbuffer < texit && T > m->t_eps) {
         if (m->dynamic_sampling) { /* gaussians_aabb.cu:267-272 */
             float dt_dist = fmaxf(tbuffer / 1024.0f, dt_base);
-            float coeff = 1.0f / cbrtf(T);
+            float coeff = (1.0f / cbrtf(T)) * g_step_scale;
             dt = fminf(dt_dist * coeff, 4.0f * dt_base);
             slab_spacing = dt * BUFFER_SIZE;
         }
@@ -747,7 +748,7 @@ static void march_backward_ray(const OrcCamera *cam, const OrcMarch *m, const fl
     while (tbuffer < texit && T > m->t_eps) {
         if (m->dynamic_sampling) {
             float dt_dist = fmaxf(tbuffer / 1024.0f, dt_base);
-            float coeff = 1.0f / cbrtf(T);
+            float coeff = (1.0f / cbrtf(T)) * g_step_scale;
             dt = fminf(dt_dist * coeff, 4.0f * dt_base);
             slab_spacing = dt * BUFFER_SIZE;
         }
@@ -944,6 +945,10 @@ int orc_num_threads(void)
     return 1;
 #endif
 }
+
+/* Sensitivity probe for the tests: scales the adaptive step's coefficient (1.0f: exactly the
+ * reference's arithmetic; 1 + 2^-23: as if cbrtf had rounded the other way). */
+void orc_set_step_scale(float s) { g_step_scale = s; }
 
 void orc_set_num_threads(int n)
 {

@@ -177,3 +177,34 @@ def test_heavy_tailed_scene_ray_sample_against_the_oracle(gx, orc):
         for k in PARAMS:
             cos, rel = gx.cos_rel(out["grads"][k], og[k])
             assert cos >= COS_MIN and rel <= rel_max, (adaptive, k, cos, rel)
+
+
+def test_tile_cooperative_and_per_ray_queries_find_the_same_hits(gx, orc, big):
+    """Two implementations of the collect query on the GPU, at the benchmark's size: the per-ray
+    skip-link traversal (rgx_trace_segments: the plain `/` and sqrtf(), pinned against the oracle on
+    small scenes) and the tile-cooperative one the march kernels use (rgx_collect_tiles: candidate
+    tables, the short division and square-root sequences).  Same segments, same hit sets, for every
+    pixel and at several depths -- some ten million ray-Gaussian hits."""
+    from raygaussx_amd import optix_utils as u_ox
+    from raygaussx_amd.render_optix import compute_rgb
+    sc, cam, cfg = big
+    d = gx.to_dev(sc)
+    gas = u_ox.AccelerationStructure(N, gx.DEV).build_from_gaussians(d["positions"], d["scales"], d["quaternions"], d["densities"])
+    eye = torch.as_tensor(np.asarray(cam.camera_center, np.float32))
+    rgb = compute_rgb(eye.to(gx.DEV), d["positions"], d["color_features"], None, None, None, 0, 3)
+    ps = u_ox.pack_prims(gas, eye, d["positions"], d["scales"], d["quaternions"], d["densities"], rgb)
+    dirs = torch.from_numpy(orc.ray_dirs(orc.camera_struct(cam))).to(gx.DEV)
+    cams = u_ox.camera_struct(cam)
+    cap, total = 128, 0
+    for t0 in (2.6, 3.4, 4.1, 5.0):
+        tlo = torch.full((W * H,), t0, dtype=torch.float32, device=gx.DEV)
+        thi = tlo + 0.08
+        _step(f"both collect queries, slab at t = {t0}")
+        c_tile, i_tile = u_ox.collect_tiles(gas, cams, ps, tlo, thi, cap)
+        c_ray, i_ray = u_ox.trace_segments(gas, ps, eye, dirs, tlo, thi, cap)
+        assert int(c_ray.min()) >= 0 and int(c_ray.max()) < cap          # no list was cut
+        assert torch.equal(c_tile, c_ray)
+        # -1 pads the unused tail of a row in both; sorted rows must agree
+        assert torch.equal(torch.sort(i_tile, dim=1).values, torch.sort(i_ray, dim=1).values)
+        total += int(c_ray.sum())
+    assert total > 5_000_000

@@ -189,11 +189,41 @@ def _march_ws(n, n_rays, max_prim_slice, device):
 REC_TILE_WORDS = 16384 + 64 * 8192
 
 
-def new_records(cam, device, tile_words=REC_TILE_WORDS):
-    """Buffer for the hit-list record of one forward launch (see rgx_march_records_bytes)."""
-    nbytes = L.size_query(L.lib().rgx_march_records_bytes, C.c_int32(cam.width), C.c_int32(cam.height),
-                          C.c_int32(tile_words))
-    return torch.empty(nbytes, dtype=torch.uint8, device=device)
+REC_LIST_WORDS = 16384        # the hit lists' share of a tile's record
+REC_SLOT_WORDS = 8192         # one slot of sample sums
+REC_MEMORY_SHARE = 0.4        # of the device's memory: the most a record may take by default
+
+
+def records_bytes(cam, tile_words):
+    return L.size_query(L.lib().rgx_march_records_bytes, C.c_int32(cam.width), C.c_int32(cam.height), C.c_int32(tile_words))
+
+
+def fit_tile_words(cam, tile_words, budget_bytes):
+    """The record size per tile that fits ``budget_bytes``: ``tile_words`` if it does; else the hit
+    lists plus as many sample-sum slots per tile as fit (tiles that find the pool empty are replayed
+    from their lists); else the hit lists alone; 0 when not even those fit (no record)."""
+    if records_bytes(cam, tile_words) <= budget_bytes:
+        return tile_words
+    lists = min(tile_words, REC_LIST_WORDS)
+    if records_bytes(cam, lists) > budget_bytes:
+        return 0
+    ntiles = ((cam.width + 7) // 8) * ((cam.height + 7) // 8)
+    slots = (budget_bytes // (4 * ntiles) - lists) // REC_SLOT_WORDS
+    return lists + slots * REC_SLOT_WORDS if (tile_words > lists and slots >= 1) else lists
+
+
+def new_records(cam, device, tile_words=REC_TILE_WORDS, budget_bytes=None):
+    """Buffer for the record of one forward launch (see rgx_march_records_bytes), or None when no
+    record fits the budget (default: REC_MEMORY_SHARE of the device's memory) or the allocator."""
+    if budget_bytes is None:
+        budget_bytes = int(REC_MEMORY_SHARE * torch.cuda.get_device_properties(device).total_memory)
+    words = fit_tile_words(cam, tile_words, budget_bytes)
+    while words:
+        try:
+            return torch.empty(records_bytes(cam, words), dtype=torch.uint8, device=device)
+        except torch.cuda.OutOfMemoryError:
+            words = REC_LIST_WORDS if words > REC_LIST_WORDS else 0   # try the hit lists alone, then give up
+    return None
 
 
 def march_forward(gas, cam, prims, dt_step, dynamic_sampling, max_prim_slice, white_background,

@@ -131,3 +131,20 @@ def test_scenes_are_seeded_and_shaped_as_the_configs_say():
     fwd = cam.world_view_transform[:3, 2]
     to_origin = -cam.camera_center / cam.camera_center.norm()
     assert float(fwd @ to_origin) > 0.999                            # look-at cameras face the scene centre
+
+
+
+def test_record_size_fits_a_memory_budget():
+    """optix_utils.fit_tile_words: the full record if it fits, else fewer sample-sum slots, else the
+    hit lists alone, else no record (host arithmetic on the library's size query)."""
+    cs = _lib.RgxCamera()
+    cs.width, cs.height = 3840, 2160                      # 129 600 tiles
+    full = u_ox.records_bytes(cs, u_ox.REC_TILE_WORDS)
+    assert full == 129600 * u_ox.REC_TILE_WORDS * 4 > 250e9
+    assert u_ox.fit_tile_words(cs, u_ox.REC_TILE_WORDS, full) == u_ox.REC_TILE_WORDS
+    w = u_ox.fit_tile_words(cs, u_ox.REC_TILE_WORDS, 100 * 2**30)
+    assert u_ox.REC_LIST_WORDS < w < u_ox.REC_TILE_WORDS and (w - u_ox.REC_LIST_WORDS) % u_ox.REC_SLOT_WORDS == 0
+    assert u_ox.records_bytes(cs, w) <= 100 * 2**30 < u_ox.records_bytes(cs, w + u_ox.REC_SLOT_WORDS)
+    assert u_ox.fit_tile_words(cs, u_ox.REC_TILE_WORDS, 10 * 2**30) == u_ox.REC_LIST_WORDS
+    assert u_ox.fit_tile_words(cs, u_ox.REC_TILE_WORDS, 2**30) == 0
+    assert u_ox.fit_tile_words(cs, 4096, 10 * 2**30) == 4096     # a caller's small record is left alone

@@ -762,3 +762,38 @@ def test_plain_division_and_square_root_are_correctly_rounded(gx):
     _lib.check(_lib.lib().rgx_check_plain_arith(_lib.ptr(tiny), _lib.ptr(huge), C.c_int64(1024), _lib.ptr(bad), _lib.stream()))
     torch.cuda.synchronize()
     assert int(bad.item()) > 0
+
+
+def test_seeded_sweep_over_scenes_image_shapes_and_settings(gx, orc):
+    """Twenty seeded draws of scene generator, Gaussian count, scale factor, SH degree, camera, ragged
+    image shape, background, max_prim_slice and record size against the oracle: counters equal and
+    the gates held wherever no hit list was cut (a cut list keeps different hits on the two sides)."""
+    rng = np.random.default_rng(2024)
+    compared = 0
+    for case in range(20):
+        config = int(rng.choice([0, 1, 2, 4]))
+        n = int(rng.choice([300, 2000, 8000, 25000]))
+        mult = float(rng.choice([0.5, 1.0, 2.0, 4.0, 8.0]))
+        w, h = int(rng.integers(9, 140)), int(rng.integers(9, 120))
+        cap = int(rng.choice([16, 64, 2048]))
+        white = bool(rng.integers(0, 2))
+        words = [None, 16384, 16384 + 2 * 8192, 2048][int(rng.integers(0, 4))]
+        sc = scenes.scene_to_numpy(scenes.make_scene(config, n=n, sh_degree=int(rng.integers(0, 4)), seed=int(rng.integers(0, 1000))))
+        sc = {k: sc[k] for k in ("positions", "scales", "quaternions", "densities", "color_features")}
+        sc["scales"] = sc["scales"] * mult
+        cam = scenes.make_camera(config, int(rng.integers(0, 5)), width=w, height=h)
+        cfg = dict(scenes.CONFIGS[config], dynamic_sampling=False, max_prim_slice=cap)
+        img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], False, cap, white_background=white, t_eps=cfg.get("t_eps", 1e-3))
+        dloss = rng.normal(size=img.shape).astype(np.float32)
+        og, _ = orc.render_backward(sc, ctx, img, dloss)
+        _step(f"sweep case {case}: config {config}, n {n}, scales x{mult}, {w}x{h}, cap {cap}, white {white}, record {words}")
+        out = gx.gpu_render(sc, cam, cfg, white=white, want_grad=dloss, rec_tile_words=words)
+        assert (out["stats_fwd"]["overflow_rays"] > 0) == (st["overflow_rays"] > 0)
+        if st["overflow_rays"]:
+            continue
+        for k in ("hit_pairs", "slabs", "empty_slabs", "rays_hit"):
+            assert out["stats_fwd"][k] == st[k], (case, k)
+        assert np.abs(out["image"] - img).max() <= IMG_TOL
+        _check_grads(gx, out["grads"], og)
+        compared += 1
+    assert compared >= 10

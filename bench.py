@@ -186,17 +186,20 @@ def main():
         tree = u_ox.AccelerationStructure(n, dev).build_from_gaussians(dscene["positions"], dscene["scales"],
                                                                         dscene["quaternions"], dscene["densities"])
 
-    def step(i):
+    def step(i, census=False):
+        """One step.  Timed steps run the kernels as a training loop does, without a statistics block;
+        the census pass afterwards repeats the same views with one to count the hit pairs."""
         nonlocal gas
         if inference:   # per frame: view-dependent colour, primitive records, march
             cam = cams[(7 * i) % n_cams]
             rgb = compute_rgb(cam.camera_center, dscene["positions"], dscene["color_features"], None, None, None, 0, 3)
             return u_ox.launch_pipeline_test(None, None, tree, None, None, cfg["dt_step"], cfg["dynamic_sampling"], cam,
                                              dscene["densities"], rgb, dscene["positions"], dscene["scales"],
-                                             dscene["quaternions"], cfg["max_prim_slice"], t_eps=cfg["t_eps"], stats=stats)
+                                             dscene["quaternions"], cfg["max_prim_slice"], t_eps=cfg["t_eps"],
+                                             stats=stats if census else None)
         s = default_settings(cams[i % n_cams], cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
                              t_eps=cfg["t_eps"], gas=gas)
-        s.stats = stats
+        s.stats = stats if census else None
         s.record_hits = not args.no_records
         if args.rec_tile_words is not None:
             s.rec_tile_words = args.rec_tile_words
@@ -212,7 +215,6 @@ def main():
     for i in range(args.warmup):
         step(i)
     torch.cuda.synchronize()
-    stats.zero_()
     L.timing_enable(True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -222,6 +224,9 @@ def main():
     elapsed = time.perf_counter() - t0
     timing = L.timing_read()
     L.timing_enable(False)
+    for i in range(args.steps):     # census: the same views once more, counted, not timed
+        step(args.warmup + i, census=True)
+    torch.cuda.synchronize()
     st = u_ox.read_stats(stats)
 
     ms_per_step = elapsed / args.steps * 1e3

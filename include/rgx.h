@@ -158,7 +158,8 @@ int rgx_march_records_bytes(int32_t width, int32_t height, int32_t tile_words, s
  * 503-601) and the OptiX programs of cuda_train/forward/gaussians_aabb.cu:
  * ray_colors (W*H,3), row-major pixels.  cam, march: host structs.
  * prims: from rgx_pack_prims with the same ws.  records (16-byte aligned, may be NULL):
- * where to write the hit-list record.  stats may be NULL. */
+ * where to write the hit-list record.  stats may be NULL, and should be outside diagnostics:
+ * a launch without a statistics block runs kernels that carry no counters (5 % faster). */
 int rgx_march_forward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims,
                       int64_t n, float *ray_colors, void *march_ws, size_t march_ws_bytes,
                       void *records, size_t records_bytes, RgxStats *stats, void *stream);

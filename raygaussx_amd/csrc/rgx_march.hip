@@ -72,12 +72,27 @@ struct MarchParams {
     int32_t sum_slots;      // slots in the pool
 };
 
+// Launch statistics (RgxStats).  Kernels launched without a statistics block carry none of it:
+// the counters live in registers for the whole march, and the march has none to spare.
 struct Counters {
     unsigned hit_pairs = 0, slabs = 0, empty = 0, overflow = 0, rays_hit = 0;
     unsigned long long nodes = 0;
     unsigned cands = 0, cands_hit = 0; // per wave (lane 0 counts)
     unsigned replay_lost = 0;          // per wave: the backward's replay did not consume its record exactly
 };
+struct NoCount { // accepts what the kernels do to a counter, keeps nothing
+    template <typename T>
+    __device__ __forceinline__ NoCount &operator+=(T) { return *this; }
+    template <typename T>
+    __device__ __forceinline__ NoCount &operator=(T) { return *this; }
+    __device__ __forceinline__ NoCount &operator++() { return *this; }
+    __device__ __forceinline__ NoCount &operator++(int) { return *this; }
+};
+struct NoCounters {
+    NoCount hit_pairs, slabs, empty, overflow, rays_hit, nodes, cands, cands_hit, replay_lost;
+};
+template <bool STATS>
+using CountersFor = typename std::conditional<STATS, Counters, NoCounters>::type;
 
 // ---------------------------------------------------------------------------
 // wave-wide reductions with DPP (all 64 lanes must be active)
@@ -114,7 +129,8 @@ __device__ __forceinline__ float wave_max_all(float v) { return -wave_min_all(-v
 //
 // First-hit query: optixTrace with SBT offset 0 (gaussians_aabb.cu:234-247, 300-313),
 // __closesthit__ch / __miss__ms_ch (370-380).  Smallest reported t, or -1.
-__device__ float first_hit(const MarchParams &P, f3 o, f3 dir, float tlo, float thi, Counters &cn)
+template <typename Cn>
+__device__ float first_hit(const MarchParams &P, f3 o, f3 dir, float tlo, float thi, Cn &cn)
 {
     const RayBox rb = make_raybox(o, dir, thi);
     float best = -1.0f;
@@ -159,8 +175,9 @@ struct HitList {
 
 // Collect query, one ray at a time: optixTrace with SBT offset 1 + __anyhit__ah
 // (gaussians_aabb.cu:282-295, 349-367).  Used by the segment test hook.
+template <typename Cn>
 __device__ int collect(const MarchParams &P, f3 o, f3 dir, float tlo, float thi, int cap, const HitList &hl, bool &overflow,
-                       Counters &cn)
+                       Cn &cn)
 {
     const RayBox rb = make_raybox(o, dir, thi);
     int p0 = 0;
@@ -388,8 +405,9 @@ __device__ __forceinline__ void frustum_cut(const MarchParams &P, Frustum &F, fl
 
 // Fills the table from the sweep; returns the number of entries.  done: the sweep is finished;
 // plain: every entry passed plain_roots().
+template <typename Cn>
 __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int32_t *s_queue, int32_t *s_leafq, float *s_tab,
-                          bool &done, bool &plain, Counters &cn)
+                          bool &done, bool &plain, Cn &cn)
 {
     plain = true;
     const int lane = threadIdx.x;
@@ -543,6 +561,7 @@ __device__ __forceinline__ bool tile_origin(const MarchParams &P, int &px0, int 
     return tx < P.tiles_x && ty < P.tiles_y;
 }
 
+__device__ __forceinline__ void flush_stats(RgxStats *, const NoCounters &) {}
 __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
 {
     if (!st) return;
@@ -636,7 +655,8 @@ __device__ __forceinline__ bool slab_begin(const MarchParams &P, RayState &R, fl
 // End of an iteration.  Marching ray: step to the next slab; after an empty slab start searching
 // from there (gaussians_aabb.cu:297-319, 324).  Searching ray: `found` (< 0: nothing in
 // [tbuffer, searched_to]) either restarts the march at the hit or moves the search on.
-__device__ __forceinline__ void slab_end(RayState &R, bool need, int p0, float found, float searched_to, Counters &cn)
+template <typename Cn>
+__device__ __forceinline__ void slab_end(RayState &R, bool need, int p0, float found, float searched_to, Cn &cn)
 {
     if (!R.active) return;
     if (R.searching) {
@@ -786,9 +806,9 @@ struct LaneQuery {
 // PART (the same for all lanes): 0: all hits of [tlo, thi]; 1: only those reaching the first 16
 // samples; 2: only those reaching the second 16, of which the ones that also reach the first are
 // not counted again.  PLAIN: every entry of the table passed plain_roots().
-template <bool SEARCH, int PART, bool PLAIN>
+template <bool SEARCH, int PART, bool PLAIN, typename Cn>
 __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, float t1, const LaneQuery &Q, int &p0, bool &ov,
-                                             float &found, int &len, Counters &cn)
+                                             float &found, int &len, Cn &cn)
 {
     const int lane = threadIdx.x, row = lane >> 4;
     len = 0;
@@ -1236,10 +1256,10 @@ __device__ __forceinline__ void frustum_range(Frustum &F, float t0, float t1)
 // row lists in lock step (it sums over the rays of a row).  WALK_ROWS: both bodies over the row lists.
 // Returns the phase-1 participation flag of this lane.
 enum { WALK_FORWARD, WALK_BACKWARD, WALK_ROWS };
-template <int WALK, typename Rec, typename BodyA, typename Mid, typename BodyB>
+template <int WALK, typename Cn, typename Rec, typename BodyA, typename Mid, typename BodyB>
 __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds &L, Frustum &F, Window &Wn, const RayState &R,
                                             bool need, float tlo, float thi, int &p0, bool &ov, float &found, float &searched_to,
-                                            Counters &cn, Rec &rec, BodyA body_a, Mid mid, BodyB body_b)
+                                            Cn &cn, Rec &rec, BodyA body_a, Mid mid, BodyB body_b)
 {
     const bool srch = R.active && R.searching, want = need || srch;
     const float t0 = wave_min_all(want ? tlo : INFINITY), t1 = wave_max_all(want ? thi : -INFINITY);
@@ -1491,7 +1511,7 @@ __device__ __forceinline__ uint8_t quantize8(float x)
 // colorBlendingT_chunked (182-203).  VIEWER: the interactive viewer's variant of the same march
 // (cuda_gui/gaussians_aabb.cu): black background, uchar4 colours, and the expected depth
 // sum T (1 - w) t over the samples (its colorBlendingT_chunked, 183-205).
-template <bool RECORD, bool VIEWER>
+template <bool RECORD, bool VIEWER, bool STATS>
 __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchParams P)
 {
     RGX_TILE_LDS();
@@ -1502,7 +1522,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
     int px, py;
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
-    Counters cn;
+    CountersFor<STATS> cn;
     Frustum F;
     frustum_planes(P.cam, px0, py0, F);
     RayState R;
@@ -1653,7 +1673,7 @@ __device__ __forceinline__ float row_sum(float v)
 // is the mask the forward blended with.  Per Gaussian the moments turn into 13 sums in its whitened
 // frame (RGX_NSUM); those are summed over the 16 rays of a row with DPP adds and carried on by one
 // lane per row; the change of variables to the 14 gradient words comes after all sums.
-template <bool REPLAY, bool SUMS>
+template <bool REPLAY, bool SUMS, bool STATS>
 __device__ __forceinline__ void march_bwd(const MarchParams &P)
 {
     static_assert(REPLAY || !SUMS, "sample sums come with a record");
@@ -1679,7 +1699,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
     int px, py;
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
-    Counters cn;
+    CountersFor<STATS> cn;
     RayState R;
     // a replay follows the forward's iteration sequence, so it takes the forward's conventions
     // (reciprocal multiply in the bbox test, clipped slab bounds)
@@ -1923,9 +1943,12 @@ __global__ __launch_bounds__(256) void k_tile_order(const MarchParams P)
 
 // The backward that searches the tree, and the one that replays the forward's record.  (Three
 // waves per SIMD with some spilling measured faster for the replay than two waves without.)
-__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchParams P) { march_bwd<false, false>(P); }
-__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay(const MarchParams P) { march_bwd<true, false>(P); }
-__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay_sums(const MarchParams P) { march_bwd<true, true>(P); }
+template <bool STATS>
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchParams P) { march_bwd<false, false, STATS>(P); }
+template <bool STATS>
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay(const MarchParams P) { march_bwd<true, false, STATS>(P); }
+template <bool STATS>
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay_sums(const MarchParams P) { march_bwd<true, true, STATS>(P); }
 
 // Test hook for the cooperative collect: per pixel a segment [tlo, thi] (thi < tlo = pixel idle);
 // writes each ray's hit count (negated when cut at cap) and the INPUT indices of its hits.
@@ -2140,9 +2163,11 @@ extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const Rgx
     void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
     if (P.records) {
         if (P.sum_pool) hipLaunchKernelGGL(k_zero4, dim3(1), dim3(64), 0, (hipStream_t)stream, (float4 *)P.sum_next, (int64_t)1);
-        hipLaunchKernelGGL((k_march_fwd<true, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+        if (stats) hipLaunchKernelGGL((k_march_fwd<true, false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+        else hipLaunchKernelGGL((k_march_fwd<true, false, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     } else {
-        hipLaunchKernelGGL((k_march_fwd<false, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+        if (stats) hipLaunchKernelGGL((k_march_fwd<false, false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+        else hipLaunchKernelGGL((k_march_fwd<false, false, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     }
     rgx_span_end(span, (hipStream_t)stream);
     RGX_LAUNCH_CHECK();
@@ -2159,7 +2184,8 @@ extern "C" int rgx_march_viewer(const void *ws, const RgxCamera *cam, const RgxM
     P.frame = frame;
     P.depth = depth;
     void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
-    hipLaunchKernelGGL((k_march_fwd<false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    if (stats) hipLaunchKernelGGL((k_march_fwd<false, true, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    else hipLaunchKernelGGL((k_march_fwd<false, true, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     rgx_span_end(span, (hipStream_t)stream);
     RGX_LAUNCH_CHECK();
     return RGX_OK;
@@ -2188,12 +2214,18 @@ extern "C" int rgx_march_backward(const void *ws, const RgxCamera *cam, const Rg
             hipLaunchKernelGGL(k_tile_order, dim3(8), dim3(256), 0, s, P);
             P.use_tile_order = 1;
         }
-        if (P.sum_pool) hipLaunchKernelGGL(k_march_bwd_replay_sums, march_grid(P), dim3(64), 0, s, P);
-        hipLaunchKernelGGL(k_march_bwd_replay, march_grid(P), dim3(64), 0, s, P);
+        if (stats) {
+            if (P.sum_pool) hipLaunchKernelGGL(k_march_bwd_replay_sums<true>, march_grid(P), dim3(64), 0, s, P);
+            hipLaunchKernelGGL(k_march_bwd_replay<true>, march_grid(P), dim3(64), 0, s, P);
+        } else {
+            if (P.sum_pool) hipLaunchKernelGGL(k_march_bwd_replay_sums<false>, march_grid(P), dim3(64), 0, s, P);
+            hipLaunchKernelGGL(k_march_bwd_replay<false>, march_grid(P), dim3(64), 0, s, P);
+        }
         P.only_overflow = 1;
         P.use_tile_order = 0;
     }
-    hipLaunchKernelGGL(k_march_bwd, march_grid(P), dim3(64), 0, s, P);
+    if (stats) hipLaunchKernelGGL(k_march_bwd<true>, march_grid(P), dim3(64), 0, s, P);
+    else hipLaunchKernelGGL(k_march_bwd<false>, march_grid(P), dim3(64), 0, s, P);
     rgx_span_end(span, s);
     span = rgx_span_begin(RGX_T_UNPERMUTE, s);
     hipLaunchKernelGGL(k_unpermute_grads, grid_for(n, 256), dim3(256), 0, s, (const float4 *)P.gbuf, P.order, n, ddens, drgb,

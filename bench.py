@@ -39,8 +39,8 @@ HBM_PEAK_GBPS = 8000.0
 # script scaled by a 1 GiB copy (--calibrate-copy); the counter readings are kept in
 # profiles/march_kernels_c4_1M_800x800.md.  Workloads without a measurement report null.
 MEASURED_TRAFFIC_BYTES = {
-    ("c4_1M_800x800", "march_backward"): 18.2e9,   # k_march_bwd_replay_sums: 14.9 GB read (14.0 the sample sums), 3.3 GB written
-    ("c4_1M_800x800", "march_forward"): 17.4e9,    # k_march_fwd<true, false>: 2.3 GB read, 15.1 GB written (14.0 the sample sums)
+    ("c4_1M_800x800", "march_backward"): 17.3e9,   # k_march_bwd_replay_sums<false>: 14.7 GB read (14.0 the sample sums), 2.6 GB written
+    ("c4_1M_800x800", "march_forward"): 15.6e9,    # k_march_fwd<true, false, false>: 1.3 GB read, 14.4 GB written (14.0 the sample sums)
 }
 
 WORKLOADS = {

@@ -528,6 +528,10 @@ def test_viewer_frame_depth_and_strided_colours(gx, orc, c0):
                          torch.from_numpy(ctx["rgb"]).to(gx.DEV))
     _step("viewer march")
     f_gpu, z_gpu = u_ox.march_viewer(gas, u_ox.camera_struct(cam), ps, cfg["dt_step"], False, cfg["max_prim_slice"])
+    # the same launch with a statistics block runs the counting variant of the kernel: same frame
+    st_v = u_ox.new_stats(gx.DEV)
+    f_cnt, z_cnt = u_ox.march_viewer(gas, u_ox.camera_struct(cam), ps, cfg["dt_step"], False, cfg["max_prim_slice"], stats=st_v)
+    assert torch.equal(f_cnt, f_gpu) and torch.equal(z_cnt, z_gpu) and u_ox.read_stats(st_v)["hit_pairs"] == st["hit_pairs"]
     f_gpu, z_gpu = f_gpu.cpu().numpy().reshape(-1, 4), z_gpu.cpu().numpy().reshape(-1)
     assert (depth > 0).sum() > 5000
     assert np.abs(z_gpu - depth).max() <= 1e-4 * depth.max()

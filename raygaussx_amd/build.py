@@ -5,6 +5,12 @@
 evaluation (fused multiply-adds only where the source says fmaf);
 ``-munsafe-fp-atomics`` selects the hardware fp32 atomic add for the gradient
 scatter; packed-fp32 code generation is disabled.
+
+``python -m raygaussx_amd.build --resources`` also prints what every kernel takes: registers,
+bytes of register spills per lane, LDS.  The march kernels are sized for three wavefronts per SIMD
+(168 registers) and twelve tiles per CU (12 800 bytes of LDS); a change that pushes spills into
+their sweep loops costs more than most optimisations gain, so look at this table after touching
+them.
 """
 import os
 import subprocess
@@ -19,10 +25,37 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
          "-Wno-unused-command-line-argument"]
 
 
-def build(verbose=False, extra=(), lib=LIB, tag=""):
-    """``extra``: more hipcc flags; ``lib`` / ``tag``: write a differently named library and objects."""
+def _resource_table(compiler_output):
+    """Kernel name, VGPRs, spill bytes per lane, waves per SIMD, LDS bytes from -Rpass-analysis remarks."""
+    rows, cur = [], None
+    for line in compiler_output.splitlines():
+        if "remark:" not in line:
+            continue
+        text = line.split("remark:", 1)[1].strip()
+        key, _, val = text.partition(":")
+        val = val.split("[")[0].strip()
+        if key.strip() == "Function Name":
+            cur = {"name": val}
+            rows.append(cur)
+        elif cur is not None and key.strip() in ("VGPRs", "ScratchSize [bytes/lane]", "Occupancy [waves/SIMD]", "LDS Size [bytes/block]"):
+            cur[key.strip()] = val
+    seen, out = set(), []
+    for r in rows:     # the host pass repeats the device pass's remarks
+        if r["name"] in seen or "VGPRs" not in r:
+            continue
+        seen.add(r["name"])
+        out.append(f"{r['name'][:70]:70s} vgpr {r.get('VGPRs', '?'):>4s}  spill B/lane {r.get('ScratchSize [bytes/lane]', '?'):>4s}  "
+                   f"waves/SIMD {r.get('Occupancy [waves/SIMD]', '?'):>2s}  LDS {r.get('LDS Size [bytes/block]', '?'):>6s}")
+    return "\n".join(out)
+
+
+def build(verbose=False, extra=(), lib=LIB, tag="", resources=False):
+    """``extra``: more hipcc flags; ``lib`` / ``tag``: write a differently named library and objects;
+    ``resources``: print every kernel's register, spill and LDS use."""
     objs = []
     procs = []
+    if resources:
+        extra = [*extra, "-Rpass-analysis=kernel-resource-usage"]
     for src in SOURCES:
         obj = os.path.join(CSRC, src.replace(".hip", tag + ".o"))
         cmd = ["hipcc", *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
@@ -37,6 +70,8 @@ def build(verbose=False, extra=(), lib=LIB, tag=""):
         if p.returncode != 0:
             failed = True
             print(out, file=sys.stderr)
+        elif resources:
+            print(f"-- {src}\n{_resource_table(out)}", flush=True)
         elif verbose and out.strip():
             print(out)
     if failed:
@@ -47,4 +82,4 @@ def build(verbose=False, extra=(), lib=LIB, tag=""):
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build(verbose=True, resources="--resources" in sys.argv[1:]))

@@ -142,6 +142,9 @@ def main():
     ap.add_argument("--rec-tile-words", type=int, default=None,
                     help="record size per tile in 32-bit words (16384: hit lists only, no per-sample sums); "
                          "default: the renderer's own")
+    ap.add_argument("--in-flight", type=int, default=2,
+                    help="after the timed steps, time the same steps again with this many views in flight, each on "
+                         "a stream of its own (reported beside the headline figure; 1 = skip)")
     ap.add_argument("--side-kernels", action="store_true",
                     help="time the entry points around the march (image epilogue, reorder gather, distCUDA2, viewer launch) "
                          "instead of the training step; one JSON line")
@@ -186,10 +189,17 @@ def main():
         tree = u_ox.AccelerationStructure(n, dev).build_from_gaussians(dscene["positions"], dscene["scales"],
                                                                         dscene["quaternions"], dscene["densities"])
 
-    def step(i, census=False):
+    def step(i, census=False, lane=None):
         """One step.  Timed steps run the kernels as a training loop does, without a statistics block;
-        the census pass afterwards repeats the same views with one to count the hit pairs."""
+        the census pass afterwards repeats the same views with one to count the hit pairs.  ``lane``:
+        (stream, one-element list holding that stream's tree) for the views-in-flight pass."""
         nonlocal gas
+        if lane is not None:
+            with torch.cuda.stream(lane[0]):
+                keep, gas = gas, lane[1][0]
+                out = step(i)
+                lane[1][0], gas = gas, keep
+            return out
         if inference:   # per frame: view-dependent colour, primitive records, march
             cam = cams[(7 * i) % n_cams]
             rgb = compute_rgb(cam.camera_center, dscene["positions"], dscene["color_features"], None, None, None, 0, 3)
@@ -228,6 +238,21 @@ def main():
         step(args.warmup + i, census=True)
     torch.cuda.synchronize()
     st = u_ox.read_stats(stats)
+    in_flight = None
+    if args.in_flight > 1:     # views of one accumulation window are independent: keep several in flight
+        lanes = [(torch.cuda.Stream(dev), [None]) for _ in range(args.in_flight)]
+        for i in range(max(args.warmup, args.in_flight)):
+            step(i, lane=lanes[i % len(lanes)])
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step(args.warmup + i, lane=lanes[i % len(lanes)])
+        torch.cuda.synchronize()
+        el = time.perf_counter() - t0
+        in_flight = dict(views=args.in_flight, value=round(n_rays * args.steps / el / 1e6, 4), unit="Mrays/s",
+                         ms_per_step=round(el / args.steps * 1e3, 4))
+        if inference:
+            in_flight["frames_per_s"] = round(args.steps / el, 3)
 
     ms_per_step = elapsed / args.steps * 1e3
     mrays = n_rays * args.steps / elapsed / 1e6
@@ -274,6 +299,7 @@ def main():
                stats_per_step={k: v / args.steps for k, v in st.items()})
     if inference:
         out["frames_per_s"] = round(1e3 / ms_per_step, 3)
+    out["views_in_flight"] = in_flight
     if args.cpu_rays > 0:
         threads = min(16, os.cpu_count() or 1)
         out["cpu_baseline"] = cpu_baseline(scene, scenes.make_camera(config, 0, width=width, height=height), cfg,

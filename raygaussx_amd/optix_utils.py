@@ -20,11 +20,13 @@ _scratch = {}
 
 
 def _workspace(key, nbytes, device):
-    """Cached byte tensor (grown, never shrunk) -- keeps the hot path free of allocations."""
-    t = _scratch.get((key, device))
+    """Cached byte tensor (grown, never shrunk) -- keeps the hot path free of allocations.  One per
+    stream: views rendered on different streams run concurrently and must not share scratch memory."""
+    slot = (key, device, torch.cuda.current_stream(device).cuda_stream)
+    t = _scratch.get(slot)
     if t is None or t.numel() < nbytes:
         t = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
-        _scratch[(key, device)] = t
+        _scratch[slot] = t
     return t
 
 

@@ -801,3 +801,44 @@ def test_seeded_sweep_over_scenes_image_shapes_and_settings(gx, orc):
         _check_grads(gx, out["grads"], og)
         compared += 1
     assert compared >= 10
+
+
+def test_views_in_flight_on_two_streams_equal_the_views_one_after_another(gx):
+    """A training loop that accumulates gradients over several views (scripts/train.py:119-148 with
+    gradient accumulation) may keep two views in flight, each on a stream of its own: the library's
+    scratch memory is per stream and its records are per call.  Images must be those of the serial
+    loop in every bit, and the accumulated gradients equal up to the order of the atomic adds."""
+    from raygaussx_amd.render_optix import RenderOptixFunction, default_settings
+    names = ("positions", "scales", "quaternions", "densities", "color_features")
+    scene = {k: v.to(gx.DEV) for k, v in scenes.make_scene(1, n=40000, seed=5).items()}
+    scene["scales"] = scene["scales"] * 3.0
+    cams = [scenes.make_camera(1, i, width=200, height=152).to(gx.DEV) for i in (0, 9, 31, 58, 77, 90)]
+    targets = [torch.rand(200 * 152, 3, device=gx.DEV, generator=torch.Generator(gx.DEV).manual_seed(i)) for i in range(len(cams))]
+    empty = (torch.zeros(40000, 3, 0, device=gx.DEV), torch.zeros(40000, 0, device=gx.DEV), torch.zeros(40000, 0, 3, device=gx.DEV))
+
+    def loop(streams):
+        params = [scene[k].clone().requires_grad_(True) for k in names]
+        gas = [None] * len(streams)
+        images = []
+        torch.cuda.synchronize()
+        for i, cam in enumerate(cams):
+            k = i % len(streams)
+            with torch.cuda.stream(streams[k]):
+                s = default_settings(cam, 0.005, False, 512, gas=gas[k])
+                img = RenderOptixFunction.apply(*params, *empty, s)
+                gas[k] = s.gas
+                ((img - targets[i]) ** 2).mean().backward()
+                images.append(img.detach())
+        torch.cuda.synchronize()
+        return images, [p.grad.clone() for p in params]
+
+    _step("six views, one stream")
+    img1, g1 = loop([torch.cuda.current_stream(gx.DEV)])
+    _step("six views, two in flight")
+    img2, g2 = loop([torch.cuda.Stream(gx.DEV), torch.cuda.Stream(gx.DEV)])
+    for a, b in zip(img1, img2):
+        assert torch.equal(a, b)
+    for k, a, b in zip(names, g1, g2):
+        rel = float((a - b).norm() / a.norm())
+        assert rel <= 1e-5, (k, rel)
+        assert float(a.norm()) > 0

@@ -85,6 +85,9 @@ class RenderOptixSettings:
         self.stats = None   # optional optix_utils.new_stats() block
         self.record_hits = True   # forward records its hit lists for the backward to replay
         self.rec_tile_words = u_ox.REC_TILE_WORDS   # record size per 8x8 pixel tile, 32-bit words
+        # True: ``gas`` was built from these very positions, scales, quaternions and densities (an earlier
+        # view of the same accumulation window) -- the forward then skips the rebuild
+        self.gas_is_current = False
 
 
 def default_settings(viewpoint_cam, dt_step, dynamic_sampling, max_prim_slice, num_sph_gauss=0,
@@ -106,9 +109,11 @@ class RenderOptixFunction(torch.autograd.Function):
         n, dev = positions.shape[0], positions.device
         # render_optix.py:109-117: boxes + acceleration structure (rebuilt unless settings.update)
         gas = settings.gas
-        if gas is None or not isinstance(gas, u_ox.AccelerationStructure) or gas.n != n or gas.device != dev:
+        stale = gas is None or not isinstance(gas, u_ox.AccelerationStructure) or gas.n != n or gas.device != dev
+        if stale:
             gas = u_ox.AccelerationStructure(n, dev)
-        gas.build_from_gaussians(positions, scales, normalized_quaternions, densities)
+        if stale or not settings.gas_is_current:
+            gas.build_from_gaussians(positions, scales, normalized_quaternions, densities)
         settings.gas = gas
         order_sh = int(round(math.sqrt(color_features.shape[2]))) - 1   # render_optix.py:119
         cam = u_ox.camera_struct(settings.viewpoint_cam, settings.supersampling)

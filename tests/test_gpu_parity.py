@@ -842,3 +842,43 @@ def test_views_in_flight_on_two_streams_equal_the_views_one_after_another(gx):
         rel = float((a - b).norm() / a.norm())
         assert rel <= 1e-5, (k, rel)
         assert float(a.norm()) > 0
+
+
+def test_a_tree_marked_current_is_not_rebuilt_and_gives_the_same_view(gx):
+    """``settings.gas_is_current``: the views of one accumulation window share the Gaussians, so all
+    but the first may skip the rebuild.  Same image and gradients, and no build launch."""
+    from raygaussx_amd.render_optix import RenderOptixFunction, default_settings
+    names = ("positions", "scales", "quaternions", "densities", "color_features")
+    scene = {k: v.to(gx.DEV) for k, v in scenes.make_scene(0, n=6000, seed=3).items()}
+    scene["scales"] = scene["scales"] * 2.0
+    cam = scenes.make_camera(0, 0, width=96, height=80).to(gx.DEV)
+    empty = (torch.zeros(6000, 3, 0, device=gx.DEV), torch.zeros(6000, 0, device=gx.DEV), torch.zeros(6000, 0, 3, device=gx.DEV))
+
+    def view(gas, current, src=scene):
+        params = [src[k].clone().requires_grad_(True) for k in names]
+        s = default_settings(cam, 0.01, False, 512, gas=gas)
+        s.gas_is_current = current
+        img = RenderOptixFunction.apply(*params, *empty, s)
+        (img ** 2).sum().backward()
+        torch.cuda.synchronize()
+        return img.detach(), [p.grad for p in params], s.gas
+
+    _step("rebuilt, then reused")
+    img_a, g_a, gas = view(None, False)
+    img_b, g_b, gas_b = view(gas, True)
+    assert gas_b is gas and torch.equal(img_a, img_b)
+    for a, b in zip(g_a, g_b):
+        assert float((a - b).norm() / a.norm()) <= 1e-5
+    img_c, _, _ = view(None, True)      # nothing to reuse: built regardless of the flag
+    assert torch.equal(img_a, img_c)
+    from raygaussx_amd import _lib
+    _lib.timing_enable(True)        # and the flag is honoured: no build launch for the reused view
+    try:
+        view(gas, True)
+        torch.cuda.synchronize()
+        assert _lib.timing_read()["build"][1] == 0
+        view(gas, False)
+        torch.cuda.synchronize()
+        assert _lib.timing_read()["build"][1] == 1
+    finally:
+        _lib.timing_enable(False)

@@ -882,3 +882,27 @@ def test_a_tree_marked_current_is_not_rebuilt_and_gives_the_same_view(gx):
         assert _lib.timing_read()["build"][1] == 1
     finally:
         _lib.timing_enable(False)
+
+
+def test_off_centre_principal_point_and_rolled_camera(gx, orc):
+    """COLMAP cameras carry a principal point away from the image centre (optix_utils.py:258-266 passes
+    Px, Py on; gaussians_aabb.cu:200-206 shifts the pixel grid by them).  The tile frusta that cull the
+    tree must follow that shift: counters, image and gradients against the oracle for a rolled camera
+    with the principal point well off centre, looking past the scene's middle."""
+    sc = scenes.scene_to_numpy(scenes.make_scene(0, n=5000, seed=17))
+    sc = {k: sc[k] for k in ("positions", "scales", "quaternions", "densities", "color_features")}
+    sc["scales"] = sc["scales"] * 2.0
+    rng = np.random.default_rng(4)
+    for px, py, up, target in ((0.31, 0.66, (0.3, -0.2, 1.0), (0.2, -0.1, 0.1)), (0.72, 0.4, (1.0, 0.1, 0.2), (-0.3, 0.2, 0.0))):
+        cam = scenes.look_at_camera((2.1, -2.4, 1.7), target=target, up=up, fov_x_deg=52.0, width=150, height=90, px=px, py=py)
+        cfg = dict(scenes.CONFIGS[0])
+        img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], False, cfg["max_prim_slice"], t_eps=cfg.get("t_eps", 1e-3))
+        dloss = rng.normal(size=img.shape).astype(np.float32)
+        og, _ = orc.render_backward(sc, ctx, img, dloss)
+        _step(f"principal point ({px}, {py})")
+        out = gx.gpu_render(sc, cam, cfg, want_grad=dloss)
+        assert st["rays_hit"] > 5000 and st["overflow_rays"] == 0
+        for k in ("hit_pairs", "slabs", "empty_slabs", "rays_hit"):
+            assert out["stats_fwd"][k] == st[k], k
+        assert np.abs(out["image"] - img).max() <= IMG_TOL
+        _check_grads(gx, out["grads"], og)

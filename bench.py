@@ -299,6 +299,10 @@ def main():
                stats_per_step={k: v / args.steps for k, v in st.items()})
     if inference:
         out["frames_per_s"] = round(1e3 / ms_per_step, 3)
+    if not args.forward_only:   # the gradient scatter: fp32 atomic adds to memory per backward launch (census) over its time
+        adds = st["grad_atomics"] / args.steps
+        out["atomics"] = dict(per_backward_launch=int(adds), unit="G atomic adds/s",
+                              value=round(adds / (per_kernel["march_backward"]["kernel_ms"] * 1e-3) / 1e9, 3))
     out["views_in_flight"] = in_flight
     if args.cpu_rays > 0:
         threads = min(16, os.cpu_count() or 1)

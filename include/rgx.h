@@ -28,7 +28,7 @@
 extern "C" {
 #endif
 
-#define RGX_ABI_VERSION 3
+#define RGX_ABI_VERSION 4
 
 #define RGX_OK 0
 #define RGX_EINVAL -1     /* bad argument (null pointer, negative size, unsupported degree ...) */
@@ -72,6 +72,8 @@ typedef struct RgxStats {
     unsigned long long candidates;     /* Gaussians gathered per tile and slab iteration (filter passes) */
     unsigned long long candidates_hit; /* ... of which at least one ray of the tile hit */
     unsigned long long replay_lost;    /* tiles whose backward did not consume its hit-list record exactly (expect 0) */
+    unsigned long long grad_atomics;   /* fp32 atomic adds of the backward's gradient scatter to memory (14 per Gaussian and
+                                          window when it replays a record; 14 per Gaussian, slab and 4x4 pixel row otherwise) */
 } RgxStats;
 
 int rgx_abi_version(void);

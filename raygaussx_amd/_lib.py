@@ -29,9 +29,9 @@ class RgxMarch(C.Structure):
 
 
 STATS_FIELDS = ("hit_pairs", "slabs", "empty_slabs", "overflow_rays", "rays_hit", "nodes_visited", "candidates",
-                "candidates_hit", "replay_lost")
+                "candidates_hit", "replay_lost", "grad_atomics")
 
-ABI_VERSION = 3   # RGX_ABI_VERSION of include/rgx.h
+ABI_VERSION = 4   # RGX_ABI_VERSION of include/rgx.h
 
 # every symbol include/rgx.h declares
 SYMBOLS = ("rgx_abi_version", "rgx_strerror", "rgx_last_hip_error", "rgx_aabb", "rgx_sh_forward",

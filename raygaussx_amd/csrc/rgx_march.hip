@@ -79,6 +79,7 @@ struct Counters {
     unsigned long long nodes = 0;
     unsigned cands = 0, cands_hit = 0; // per wave (lane 0 counts)
     unsigned replay_lost = 0;          // per wave: the backward's replay did not consume its record exactly
+    unsigned grad_atomics = 0;         // fp32 atomic adds to the gradient block in memory
 };
 struct NoCount { // accepts what the kernels do to a counter, keeps nothing
     template <typename T>
@@ -89,7 +90,7 @@ struct NoCount { // accepts what the kernels do to a counter, keeps nothing
     __device__ __forceinline__ NoCount &operator++(int) { return *this; }
 };
 struct NoCounters {
-    NoCount hit_pairs, slabs, empty, overflow, rays_hit, nodes, cands, cands_hit, replay_lost;
+    NoCount hit_pairs, slabs, empty, overflow, rays_hit, nodes, cands, cands_hit, replay_lost, grad_atomics;
 };
 template <bool STATS>
 using CountersFor = typename std::conditional<STATS, Counters, NoCounters>::type;
@@ -565,8 +566,9 @@ __device__ __forceinline__ void flush_stats(RgxStats *, const NoCounters &) {}
 __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
 {
     if (!st) return;
-    unsigned long long v[9] = {c.hit_pairs, c.slabs, c.empty, c.overflow, c.rays_hit, c.nodes, c.cands, c.cands_hit, c.replay_lost};
-    for (int k = 0; k < 9; ++k) {
+    unsigned long long v[10] = {c.hit_pairs, c.slabs, c.empty, c.overflow, c.rays_hit, c.nodes, c.cands, c.cands_hit, c.replay_lost,
+                                c.grad_atomics};
+    for (int k = 0; k < 10; ++k) {
         unsigned long long x = v[k];
         for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
         v[k] = x;
@@ -576,6 +578,7 @@ __device__ __forceinline__ void flush_stats(RgxStats *st, const Counters &c)
         atomicAdd(&st->overflow_rays, v[3]); atomicAdd(&st->rays_hit, v[4]); atomicAdd(&st->nodes_visited, v[5]);
         atomicAdd(&st->candidates, v[6]); atomicAdd(&st->candidates_hit, v[7]);
         if (v[8]) atomicAdd(&st->replay_lost, v[8]);
+        if (v[9]) atomicAdd(&st->grad_atomics, v[9]);
     }
 }
 
@@ -1839,8 +1842,13 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                 for (int c = 0; c < RGX_NSUM; ++c) out[c] = row_sum(out[c]);
                 if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
                     if constexpr (REPLAY) {
-                        // to the window's sums in LDS
-                        atomicOr(&s_pid[e.slot], RGX_SLOT_TOUCHED);
+                        // to the window's sums in LDS; a slot's first touch is what replay_flush()
+                        // later turns into 14 adds to memory
+                        if constexpr (STATS) {
+                            if (!(atomicOr(&s_pid[e.slot], RGX_SLOT_TOUCHED) & RGX_SLOT_TOUCHED)) cn.grad_atomics += 14;
+                        } else {
+                            atomicOr(&s_pid[e.slot], RGX_SLOT_TOUCHED);
+                        }
 #pragma unroll
                         for (int c = 0; c < RGX_NSUM; ++c) unsafeAtomicAdd(&s_acc[c * RGX_CCAP + e.slot], out[c]);
                     } else {
@@ -1850,6 +1858,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                         float *dst = P.gbuf + (int64_t)pid * 16;
 #pragma unroll
                         for (int c = 0; c < 14; ++c) unsafeAtomicAdd(dst + c, grad[c]);
+                        cn.grad_atomics += 14;
                     }
                 }
             };

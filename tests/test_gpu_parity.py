@@ -304,6 +304,10 @@ def test_backward_replay_of_recorded_hit_lists_equals_recomputation(gx, orc):
         assert 0.9 * b["stats_fwd"]["hit_pairs"] <= a["stats_fwd"]["hit_pairs"] <= b["stats_fwd"]["hit_pairs"]
         assert a["stats_bwd"]["hit_pairs"] == b["stats_bwd"]["hit_pairs"] > 10000
         assert a["stats_bwd"]["slabs"] == b["stats_bwd"]["slabs"]
+        # gradient scatter: 14 adds per Gaussian and window when replaying, per Gaussian, slab and pixel row otherwise
+        assert a["stats_fwd"]["grad_atomics"] == b["stats_fwd"]["grad_atomics"] == 0
+        assert 0 < b["stats_bwd"]["grad_atomics"] <= a["stats_bwd"]["grad_atomics"]
+        assert a["stats_bwd"]["grad_atomics"] % 14 == b["stats_bwd"]["grad_atomics"] % 14 == 0
         if words is None or words >= 16384:   # everything replayed: the backward fetched no tree node
             assert b["stats_bwd"]["nodes_visited"] == 0
         else:               # some tiles replayed, some recomputed

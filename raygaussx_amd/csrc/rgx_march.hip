@@ -722,7 +722,12 @@ __device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, f
     const f3 Pc = mk3(fmaf(b_inv_a, De.x, Oe.x), fmaf(b_inv_a, De.y, Oe.y), fmaf(b_inv_a, De.z, Oe.z));
     const float d2 = fmaf(Pc.x, Pc.x, fmaf(Pc.y, Pc.y, Pc.z * Pc.z));
     const float disc = 1.0f - d2;
-    // no branch: where the line misses (disc <= 1e-7) the roots are garbage and the result false
+    // an entry whose ellipsoid the lines of all 64 rays miss needs no roots
+    if (!__any(disc > 1e-7f)) {
+        r1 = r2 = 0.f;
+        return false;
+    }
+    // no branch per lane: where the line misses (disc <= 1e-7) the roots are garbage and the result false
     const float sdisc = PLAIN ? sqrt_rn_plain(disc * a) : sqrtf(disc * a);
     const float q = b + copysignf(sdisc, b);
     r1 = PLAIN ? div_rn_plain(c, q) : c / q;
@@ -840,6 +845,7 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
             // straight-line code: every lane evaluates both queries' predicates, its state selects
             float r1, r2;
             const bool ok = lane_roots<PLAIN>((const float4 *)(L.tab + c * RGX_TAB), Q.dir, r1, r2);
+            if (!__any(ok)) continue;
             // first-hit query (searching lanes): smallest max(slo, r1) over the entries hit in [slo, shi]
             if constexpr (SEARCH) {
                 const float ts = fmaxf(Q.slo, r1);

@@ -707,8 +707,9 @@ struct TileLds {
 
 // Ray-interval-independent half of __intersection__gaussian (gaussians_aabb.cu:43-82) on a table
 // entry: same arithmetic as line_roots(), with the precomputed ray-independent parts.  PLAIN: the
-// entry passed plain_roots().
-template <bool PLAIN>
+// entry passed plain_roots().  EXIT: return early (false for every lane, roots zero) when no
+// lane's line meets the ellipsoid.
+template <bool PLAIN, bool EXIT>
 __device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, float &r2)
 {
     const float4 e0 = e[0], e1 = e[1], e2 = e[2], e3 = e[3], e4 = e[4];
@@ -722,10 +723,12 @@ __device__ __forceinline__ bool lane_roots(const float4 *e, f3 dir, float &r1, f
     const f3 Pc = mk3(fmaf(b_inv_a, De.x, Oe.x), fmaf(b_inv_a, De.y, Oe.y), fmaf(b_inv_a, De.z, Oe.z));
     const float d2 = fmaf(Pc.x, Pc.x, fmaf(Pc.y, Pc.y, Pc.z * Pc.z));
     const float disc = 1.0f - d2;
-    // an entry whose ellipsoid the lines of all 64 rays miss needs no roots
-    if (!__any(disc > 1e-7f)) {
-        r1 = r2 = 0.f;
-        return false;
+    // EXIT: an entry whose ellipsoid the lines of all 64 rays miss needs no roots
+    if constexpr (EXIT) {
+        if (!__any(disc > 1e-7f)) {
+            r1 = r2 = 0.f;
+            return false;
+        }
     }
     // no branch per lane: where the line misses (disc <= 1e-7) the roots are garbage and the result false
     const float sdisc = PLAIN ? sqrt_rn_plain(disc * a) : sqrtf(disc * a);
@@ -844,8 +847,12 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
             m &= m - 1;
             // straight-line code: every lane evaluates both queries' predicates, its state selects
             float r1, r2;
-            const bool ok = lane_roots<PLAIN>((const float4 *)(L.tab + c * RGX_TAB), Q.dir, r1, r2);
-            if (!__any(ok)) continue;
+            // (the counting kernels go without the early exit: it costs their recording variant its registers)
+            constexpr bool EXIT = std::is_same<Cn, NoCounters>::value;
+            const bool ok = lane_roots<PLAIN, EXIT>((const float4 *)(L.tab + c * RGX_TAB), Q.dir, r1, r2);
+            if constexpr (EXIT) {
+                if (!__any(ok)) continue;
+            }
             // first-hit query (searching lanes): smallest max(slo, r1) over the entries hit in [slo, shi]
             if constexpr (SEARCH) {
                 const float ts = fmaxf(Q.slo, r1);

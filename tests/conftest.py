@@ -12,6 +12,14 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
 
 
+def pytest_sessionstart(session):
+    """A fresh checkout has no librgx.so (built files are not in the history): compile it once.
+    The tests load what is built; they never build over an existing library."""
+    from raygaussx_amd import build
+    if not os.path.exists(build.LIB):
+        build.build()
+
+
 @pytest.fixture(scope="session")
 def orc():
     """The CPU oracle (built on demand from oracle/rgx_oracle.c)."""

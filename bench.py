@@ -15,6 +15,10 @@ upper-hemisphere orbit per step.  Inputs are resident in HBM before the timed re
 Prints ONE JSON line.  ``roofline`` prices the dominant kernel (the backward march) with its
 algorithmic bytes (64+56 B per ray-slab-hit + 24 B per ray) over its own HIP-event time;
 ``cpu_baseline`` times the CPU oracle on a bounded ray sample of the same workload.
+Beside the contract's keys: ``atomics`` (the gradient scatter's atomic adds per backward launch,
+counted by the kernels, over the launch's time) and ``views_in_flight`` (the same steps timed once
+more with two views in flight on two streams, as a loop that accumulates gradients over several
+views can run them; ``value`` itself is always one view at a time).
 """
 import argparse
 import json

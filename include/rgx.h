@@ -4,8 +4,10 @@
  *
  * Every entry point replaces a piece of the reference's OptiX/CuPy host glue
  * (paths relative to the reference tree).  Conventions:
- *   - all pointers are DEVICE pointers on the current HIP device unless the
- *     parameter is documented as "host";
+ *   - all pointers are DEVICE pointers unless the parameter is documented as
+ *     "host"; every entry point that launches work makes the device that owns
+ *     its first device pointer current for the duration of the call (and
+ *     restores the caller's), so a binding need not call hipSetDevice itself;
  *   - `stream` is a hipStream_t passed as void* (0 = the null stream); every
  *     call only enqueues work on it and never synchronises, except the two
  *     explicitly synchronous read-back helpers;
@@ -28,7 +30,7 @@
 extern "C" {
 #endif
 
-#define RGX_ABI_VERSION 4
+#define RGX_ABI_VERSION 5
 
 #define RGX_OK 0
 #define RGX_EINVAL -1     /* bad argument (null pointer, negative size, unsupported degree ...) */
@@ -126,6 +128,14 @@ int rgx_build_aabbs(const float *bboxes, int64_t n, void *ws, size_t ws_bytes, v
 int rgx_scene_bbox(const void *ws, float *host_out6, void *stream);
 /* The build's permutation: order[j] = input index of the j-th Gaussian in Morton order. */
 int rgx_build_order(const void *ws, int64_t n, int32_t *order_out, void *stream);
+/* Test hook: where a built workspace keeps the tree, as byte offsets from `ws` (host out[6]):
+ * 0 boxes (n,6) floats in input order; 1 order (n) uint32; 2 nodes (2n-1) records of 32 bytes
+ * {lo[3], left | ~sorted leaf index, hi[3], skip}, internal nodes first, leaf j of the Morton
+ * order at n-1+j; 3 parent (2n-1) int32; 4 right child (n-1) int32; 5 the 64-byte header
+ * {bb_min[3], bb_max[3], ...}.  Lets a test read a tree back and check it on the host (child
+ * boxes inside their parent, skip links, permutation); OptiX's GAS is opaque, so the reference
+ * has no counterpart. */
+int rgx_build_layout(int64_t n, size_t *host_out6);
 
 /* Replaces the prim packing at optix_utils.py:268-304: the 64-byte PrimData record
  * (gaussians_aabb.h:7-12) of every Gaussian, written in the build's Morton order
@@ -180,6 +190,15 @@ int rgx_march_backward(const void *ws, const RgxCamera *cam, const RgxMarch *mar
                        size_t march_ws_bytes, const void *records, size_t records_bytes,
                        RgxStats *stats, void *stream);
 
+/* Launch faults that do not stop a launch, counted in the march workspace (always, with or without a
+ * statistics block) and read back here; synchronous, waits for `stream`.  host_out[0]: tiles whose
+ * replaying backward did not consume its hit-list record exactly (the gradient of such a tile is
+ * that of the iterations replayed so far); host_out[1]: sweeps of the tree that had to drop nodes
+ * because the node stack was full (cannot happen for trees of at most 2^30 leaves; counted so that
+ * it would be seen).  Both are cleared by the next rgx_march_forward / rgx_march_backward on the
+ * workspace.  A workspace with room for the gradient block only keeps no counts (zeros). */
+int rgx_march_faults(const void *march_ws, size_t march_ws_bytes, int64_t n, uint64_t *host_out2, void *stream);
+
 /* The interactive viewer's two kernels (its GL window and interop stay with the caller).
  * rgx_sh_viewer replaces gui_sh (utils/sh_utils.cu:25-119): rgx_sh_forward on tensors that keep
  * room for max_num_sh coefficients per channel and max_sg_display lobes per Gaussian, of which the
@@ -232,10 +251,12 @@ int rgx_trace_segments(const void *ws, const float *prims, int64_t n_prims, cons
 
 /* The collect query as the march kernels run it: one 8x8 pixel tile per wavefront, the
  * tile's Gaussians gathered once and tested per ray.  tlo/thi (W*H) give each pixel's
- * segment (thi < tlo: pixel idle); counts (W*H) and ids (W*H,cap) as rgx_trace_segments. */
+ * segment (thi < tlo: pixel idle); counts (W*H) and ids (W*H,cap) as rgx_trace_segments.
+ * uncounted != 0 runs the filter as the kernels launched without a statistics block compile it
+ * (with its early exit for entries that no ray's line meets); 0: as the counting kernels do. */
 int rgx_collect_tiles(const void *ws, const RgxCamera *cam, const float *prims, int64_t n_prims,
                       const float *tlo, const float *thi, int32_t cap, int32_t *counts, int32_t *ids,
-                      void *stream);
+                      int32_t uncounted, void *stream);
 
 /* Test hook for the arithmetic of the hit predicate.  Where a Gaussian's scales and distance are of
  * ordinary size the kernels form the predicate's two quotients and its square root

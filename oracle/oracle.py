@@ -209,6 +209,20 @@ def march_forward(cam_struct, march, bmin, bmax, prims, ray_ids=None, out=None):
     return out, st.as_dict()
 
 
+def march_forward_counts(cam_struct, march, bmin, bmax, prims, ray_ids=None):
+    """The forward march with its counters kept per ray: (image, counts (n,2) = slabs blended and the
+    sum of their hit-list lengths, for the rays of ``ray_ids``)."""
+    prims, bmin, bmax = _f(prims), _f(bmin), _f(bmax)
+    R = cam_struct.width * cam_struct.height
+    out = np.zeros((R, 3), np.float32)
+    ids = None if ray_ids is None else np.ascontiguousarray(ray_ids, dtype=np.int64)
+    n = R if ids is None else len(ids)
+    counts = np.zeros((n, 2), np.int64)
+    lib().orc_march_forward_counts(C.byref(cam_struct), C.byref(march), _p(bmin), _p(bmax), C.c_int64(prims.shape[0]),
+                                   _p(prims), C.c_int64(n), _p(ids), _p(out), _p(counts))
+    return out, counts
+
+
 def march_trace(cam_struct, march, bmin, bmax, prims, ray, max_slabs=4096, max_ids=1 << 20):
     """Slab-by-slab record of one ray: list of (tbuffer, dt, t_lo, t_hi, ids)."""
     prims, bmin, bmax = _f(prims), _f(bmin), _f(bmax)

@@ -30,9 +30,17 @@
  *   line/segment hit    float64 closed-form ray/ellipsoid roots, equivariance
  *   orc_first_hit / orc_trace_segments   numpy brute force in float64
  *   orc_march_forward   analytic optical depth (erf) of one isotropic Gaussian,
- *                       empty scene, compositing identity, float64 numpy march
+ *                       empty scene, compositing identity, float64 numpy march;
+ *                       its dynamic_sampling branch: a float64 march that recomputes
+ *                       every step from its own transmittance (same slab sequence,
+ *                       steps and hit sets on every ray away from a decision edge),
+ *                       and closed forms on one Gaussian (T = 1: the distance term
+ *                       exactly; T(t) through erf; the 4 dt0 cap exactly)
  *   orc_march_backward  torch.autograd through a float64 torch forward with
- *                       frozen hit sets and cut-off masks + central differences
+ *                       frozen hit sets and cut-off masks + central differences;
+ *                       its dynamic_sampling branch: autograd is fed the forward's
+ *                       (pinned) slab sequence, so a backward that stepped
+ *                       differently would miss its gradients
  *   orc_march_gui       float64 quadrature of int t sigma exp(-tau) dt for one Gaussian,
  *                       depth / (1 - T) inside the scene box, known quantisation values
  *   orc_morton_codes    naive per-bit loop
@@ -623,6 +631,31 @@ void orc_march_forward(const OrcCamera *cam, const OrcMarch *m, const float *bmi
         free(ids); free(L.c);
     }
     if (stats) *stats = total;
+}
+
+/* orc_march_forward with the march counters kept per ray: counts (n,2) = slabs blended and the
+ * sum of their hit-list lengths, for the n rays of ray_ids (NULL = all).  Tells a test which rays
+ * marched the same slab sequence on both sides when the adaptive step makes that depend on the
+ * last bit of cbrt / exp. */
+void orc_march_forward_counts(const OrcCamera *cam, const OrcMarch *m, const float *bmin, const float *bmax,
+                              int64_t N, const float *prims, int64_t n, const int64_t *ray_ids,
+                              float *ray_colors, int64_t *counts)
+{
+    if (!ray_ids) n = (int64_t)cam->width * cam->height;
+#pragma omp parallel
+    {
+        CandList L = {0, 0, 0};
+        int32_t *ids = (int32_t *)malloc(sizeof(int32_t) * (size_t)(m->max_prim_slice > 0 ? m->max_prim_slice : 1));
+#pragma omp for schedule(dynamic, 16)
+        for (int64_t r = 0; r < n; ++r) {
+            int64_t ray = ray_ids ? ray_ids[r] : r;
+            OrcStats st; memset(&st, 0, sizeof st);
+            march_forward_ray(cam, m, bmin, bmax, N, prims, ray, &L, ids, ray_colors + 3 * ray, &st, NULL, NULL);
+            counts[2 * r] = st.slabs;
+            counts[2 * r + 1] = st.hit_pairs;
+        }
+        free(ids); free(L.c);
+    }
 }
 
 /* cuda_gui/helpers.h:45-59: clamp to [0,1], then min(uint(x * 256), 255) */

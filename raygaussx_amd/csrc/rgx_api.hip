@@ -9,6 +9,24 @@ int rgx_set_hip_error(hipError_t e)
     return RGX_EHIP;
 }
 
+DeviceScope::DeviceScope(const void *p)
+{
+    if (!p) return;
+    hipPointerAttribute_t attr;
+    if (hipPointerGetAttributes(&attr, p) != hipSuccess) {
+        (void)hipGetLastError(); // not memory the runtime knows: not an error of this call
+        return;
+    }
+    int cur = -1;
+    if (attr.type != hipMemoryTypeDevice || hipGetDevice(&cur) != hipSuccess || cur == attr.device) return;
+    if (hipSetDevice(attr.device) == hipSuccess) prev = cur;
+}
+
+DeviceScope::~DeviceScope()
+{
+    if (prev >= 0) (void)hipSetDevice(prev);
+}
+
 extern "C" int rgx_abi_version(void) { return RGX_ABI_VERSION; }
 
 extern "C" int rgx_last_hip_error(void) { return g_last_hip_error; }

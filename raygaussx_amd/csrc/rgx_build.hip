@@ -349,8 +349,10 @@ __global__ __launch_bounds__(256) void k_karras(const uint64_t *__restrict__ key
 // i covers the leaves between i and other_end[i], so its index is one of them) are met in LDS:
 // counters, and the box of whichever child arrived first.  Only the few subtree roots a workgroup
 // ends up with go on through memory, where box words travel between threads through agent-scope
-// atomic stores and loads (coherent across the XCDs' L2s without a cache write-back); the
-// workgroup-scope fences only order them against the counter.
+// atomic stores and loads, ordered against the arrival counter by an agent-scope release before the
+// counter's atomic and an agent-scope acquire after it: the thread that arrives second may run in
+// another workgroup on another XCD, so nothing narrower orders the first arriver's box stores (also
+// those it made in the LDS phase) before its count.
 __device__ __forceinline__ void st_agent(float *p, float v)
 {
     __hip_atomic_store((int *)p, __float_as_int(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -401,9 +403,9 @@ __global__ __launch_bounds__(256) void k_refit(int64_t n, Node *nodes, const int
     }
     // the rest of the way: through memory
     while (node >= 0) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         if (atomicAdd(&flags[node], 1) == 0) return; // the sibling subtree is not done yet
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         const Node *a = &nodes[nodes[node].left];
         const Node *b = &nodes[right[node]];
         for (int c = 0; c < 3; ++c) {
@@ -437,6 +439,7 @@ static inline dim3 grid_for(int64_t n, int block) { return dim3((unsigned)((n + 
 extern "C" int rgx_aabb(const float *pos, const float *scale, const float *quat, const float *dens, int64_t n,
                         float sigma_threshold, float *bboxes, float *bb_min, float *bb_max, void *stream)
 {
+    const DeviceScope on_device(pos);
     if (n < 0 || (n > 0 && (!pos || !scale || !quat || !dens)) || ((bb_min == nullptr) != (bb_max == nullptr)))
         return RGX_EINVAL;
     hipStream_t s = (hipStream_t)stream;
@@ -497,6 +500,7 @@ extern "C" int rgx_build_aabbs(const float *bboxes, int64_t n, void *ws, size_t 
 static int build_impl(const float *pos, const float *scale, const float *quat, const float *dens, const float *in_boxes,
                       int64_t n, float sigma_threshold, void *ws, size_t ws_bytes, void *stream)
 {
+    const DeviceScope on_device(ws);
     if (n < 0 || n > 0x3fffffff || !ws) return RGX_EINVAL;
     const WsLayout L = rgx_ws_layout(n);
     if (ws_bytes < L.total || ((uintptr_t)ws & 255u)) return RGX_EWORKSPACE;
@@ -539,10 +543,24 @@ static int build_impl(const float *pos, const float *scale, const float *quat, c
     return RGX_OK;
 }
 
+extern "C" int rgx_build_layout(int64_t n, size_t *host_out6)
+{
+    if (n < 0 || n > 0x3fffffff || !host_out6) return RGX_EINVAL;
+    const WsLayout L = rgx_ws_layout(n);
+    host_out6[0] = L.aabb;
+    host_out6[1] = L.vals0;
+    host_out6[2] = L.nodes;
+    host_out6[3] = L.parent;
+    host_out6[4] = L.right;
+    host_out6[5] = L.header;
+    return RGX_OK;
+}
+
 // ---------------------------------------------------------------------------
 // Synchronous / small read-backs of a built workspace.
 extern "C" int rgx_scene_bbox(const void *ws, float *host_out6, void *stream)
 {
+    const DeviceScope on_device(ws);
     if (!ws || !host_out6) return RGX_EINVAL;
     const WsHeader *hdr = (const WsHeader *)ws;
     RGX_HIP(hipMemcpyAsync(host_out6, hdr->bb_min, 6 * sizeof(float), hipMemcpyDeviceToHost, (hipStream_t)stream));
@@ -558,6 +576,7 @@ __global__ __launch_bounds__(256) void k_copy_order(const uint32_t *__restrict__
 
 extern "C" int rgx_build_order(const void *ws, int64_t n, int32_t *order_out, void *stream)
 {
+    const DeviceScope on_device(ws);
     if (!ws || n < 0 || (n > 0 && !order_out)) return RGX_EINVAL;
     if (n == 0) return RGX_OK;
     const WsLayout L = rgx_ws_layout(n);
@@ -641,6 +660,7 @@ extern "C" int rgx_morton_workspace_bytes(int64_t n, size_t *bytes)
 extern "C" int rgx_morton_order(const float *pos, int64_t n, int64_t *codes, int64_t *order, void *ws, size_t ws_bytes,
                                 void *stream)
 {
+    const DeviceScope on_device(pos);
     if (n < 0 || n > 0x3fffffff || !ws || (n > 0 && !pos)) return RGX_EINVAL;
     const MortonLayout L = morton_layout(n);
     if (ws_bytes < L.total || ((uintptr_t)ws & 255u)) return RGX_EWORKSPACE;
@@ -691,6 +711,7 @@ __global__ __launch_bounds__(256) void k_gather_rows(const GatherArgs A, const i
 extern "C" int rgx_gather_rows(int32_t count, const void *const *src, void *const *dst, const int64_t *row_bytes,
                                const int64_t *order, int64_t n, void *stream)
 {
+    const DeviceScope on_device(order);
     if (count < 0 || n < 0 || (count > 0 && (!src || !dst || !row_bytes)) || (n > 0 && count > 0 && !order)) return RGX_EINVAL;
     for (int i = 0; i < count; ++i)
         if (row_bytes[i] <= 0 || (row_bytes[i] & 3) || row_bytes[i] > 0x7fffffff || ((!src[i] || !dst[i]) && n > 0) || src[i] == dst[i])
@@ -842,6 +863,7 @@ extern "C" int rgx_knn_workspace_bytes(int64_t n, size_t *bytes)
 
 extern "C" int rgx_dist2_knn3(const float *pos, int64_t n, float *mean_dist2, void *ws, size_t ws_bytes, void *stream)
 {
+    const DeviceScope on_device(pos);
     if (n < 0 || n > 0x3fffffff || !ws || (n > 0 && (!pos || !mean_dist2))) return RGX_EINVAL;
     const KnnLayout K = knn_layout(n);
     if (ws_bytes < K.total || ((uintptr_t)ws & 255u)) return RGX_EWORKSPACE;

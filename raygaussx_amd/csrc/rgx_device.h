@@ -222,6 +222,17 @@ int rgx_set_hip_error(hipError_t e);
     } while (0)
 #define RGX_LAUNCH_CHECK() RGX_HIP(hipGetLastError())
 
+// Makes the device that owns device pointer `p` current for the scope of an entry point and restores
+// the caller's device afterwards (callers on another thread, e.g. the autograd engine's, may have a
+// different current device).  A pointer the runtime does not know leaves the device as it is.
+struct DeviceScope {
+    int prev = -1;
+    explicit DeviceScope(const void *p);
+    ~DeviceScope();
+    DeviceScope(const DeviceScope &) = delete;
+    DeviceScope &operator=(const DeviceScope &) = delete;
+};
+
 // Event-timed spans (rgx_timing_* in the C ABI).  begin returns NULL when timing is off.
 enum {
     RGX_T_BUILD = 0, RGX_T_SH_FWD, RGX_T_PACK, RGX_T_MARCH_FWD, RGX_T_MARCH_BWD, RGX_T_UNPERMUTE, RGX_T_SH_BWD,

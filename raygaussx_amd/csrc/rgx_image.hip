@@ -33,6 +33,7 @@ __global__ __launch_bounds__(256) void k_reduce_supersampling(const float *__res
 extern "C" int rgx_reduce_supersampling(const float *ray_colors, int32_t width, int32_t height, int32_t factor_x,
                                         int32_t factor_y, int32_t clip, float *out, uint8_t *out8, void *stream)
 {
+    const DeviceScope on_device(ray_colors);
     if (width <= 0 || height <= 0 || factor_x <= 0 || factor_y <= 0 || !ray_colors || (!out && !out8)) return RGX_EINVAL;
     const int64_t n = (int64_t)width * height;
     hipLaunchKernelGGL(k_reduce_supersampling, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, ray_colors, width, height,

@@ -38,7 +38,12 @@
 #define RGX_KLO (RGX_CCAP / 3)       // one that stayed below this, twice as many
 #endif
 #define RGX_MASK_WORDS ((RGX_CCAP + 31) / 32) // 32-bit words of a hit mask over a row's list
-#define RGX_DFS_MARGIN 128 // above QCAP - margin the sweep pops one node at a time (depth-first)
+// Above QCAP - margin the sweep pops one node at a time (depth-first).  A breadth-first step pops
+// up to 64 nodes and pushes up to 128, so it leaves at most QCAP - margin + 64 entries; a
+// depth-first step adds at most one entry per level it descends, and a Karras tree over 63-bit
+// keys with ties broken by a 30-bit index is at most 63 + 30 = 93 deep: with a margin of 160 the
+// stack never holds more than QCAP - 96 + 93 < QCAP entries, whatever the scene.
+#define RGX_DFS_MARGIN 160
 #define RGX_LDS_HITS 32    // per-lane list of the stand-alone collect hook
 // The march kernels are sized (registers and LDS) for three wavefronts per SIMD.
 #ifndef RGX_WAVES_ATTR
@@ -70,6 +75,7 @@ struct MarchParams {
     float4 *sum_pool;       // sample-sum slots of the record (RGX_SUM_SLOT_WORDS each), or null
     uint32_t *sum_next;     // next free slot (bump counter in the record's pool header)
     int32_t sum_slots;      // slots in the pool
+    uint32_t *faults;       // march workspace: [0] replays that lost their record, [1] sweeps that dropped nodes; or null
 };
 
 // Launch statistics (RgxStats).  Kernels launched without a statistics block carry none of it:
@@ -512,9 +518,11 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
         S.lqn += __popcll(bl);
         if (inner_hit) {
             const int pos = S.qn + 2 * __popcll(bi & lt);
-            if (pos + 1 < RGX_QCAP) { // cannot fail: see RGX_DFS_MARGIN (tree depth < 128)
+            if (pos + 1 < RGX_QCAP) { // cannot fail (see RGX_DFS_MARGIN); if it did, the drop is counted, not silent
                 s_queue[pos] = right;
                 s_queue[pos + 1] = left;
+            } else if (P.faults) {
+                atomicAdd(&P.faults[1], 1u);
             }
         }
         S.qn += 2 * __popcll(bi);
@@ -1897,7 +1905,10 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
             });
         }
         replay_flush(P, RL);
-        if ((rp.lost || rp.at != rp.used) && lane == 0) cn.replay_lost = 1;
+        if ((rp.lost || rp.at != rp.used) && lane == 0) {
+            cn.replay_lost = 1;
+            if (P.faults) atomicAdd(&P.faults[0], 1u); // counted with or without a statistics block
+        }
     } else {
         RGX_TILE_LDS();
         Frustum F;
@@ -1974,6 +1985,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay_sums(con
 
 // Test hook for the cooperative collect: per pixel a segment [tlo, thi] (thi < tlo = pixel idle);
 // writes each ray's hit count (negated when cut at cap) and the INPUT indices of its hits.
+template <bool STATS>
 __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const float *__restrict__ seg_lo,
                                                       const float *__restrict__ seg_hi, int cap, int32_t *__restrict__ counts,
                                                       int32_t *__restrict__ ids)
@@ -1986,7 +1998,7 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
     const int64_t ray = (int64_t)py * P.cam.width + px;
-    Counters cn;
+    CountersFor<STATS> cn; // without counters the filter compiles in its early exit, as in the kernels a training loop runs
     Frustum F;
     frustum_planes(P.cam, px0, py0, F);
     const f3 dir = compute_ray(P.cam, (unsigned)px, (unsigned)py);
@@ -2039,6 +2051,14 @@ __global__ __launch_bounds__(256) void k_zero4(float4 *p, int64_t n4)
     if (i < n4) p[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 }
 
+// Clears the 16 bytes at a and at b (either may be null): the bump counter of the record's
+// sample-sum pool and the workspace's fault counters, at the start of a forward launch.
+__global__ __launch_bounds__(64) void k_clear2(float4 *a, float4 *b)
+{
+    if (threadIdx.x == 0 && a) *a = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (threadIdx.x == 1 && b) *b = make_float4(0.f, 0.f, 0.f, 0.f);
+}
+
 // ---------------------------------------------------------------------------
 // Test hooks: the two queries on caller-supplied segments.
 __global__ __launch_bounds__(64) void k_first_hit(const MarchParams P, f3 o, int64_t n, const float *__restrict__ dirs,
@@ -2075,13 +2095,14 @@ static inline dim3 grid_for(int64_t n, int block) { return dim3((unsigned)((n + 
 // the replaying backward.  The order's room is sized from the ray count alone (images of ordinary
 // proportions fit; a launch whose tile grid needs more runs in launch order).
 struct MarchWs {
-    size_t gbuf, order, order_words, total;
+    size_t gbuf, faults, order, order_words, total;
 };
 static inline MarchWs march_ws_layout(int64_t n, int64_t n_rays)
 {
     MarchWs L;
     L.gbuf = 0;
-    L.order = rgx_align_up((size_t)(n > 0 ? n : 1) * 16 * sizeof(float), 256);
+    L.faults = rgx_align_up((size_t)(n > 0 ? n : 1) * 16 * sizeof(float), 256); // 256 bytes: the fault counters
+    L.order = L.faults + 256;
     L.order_words = (size_t)(n_rays / 64) * 5 / 4 + 2048;
     L.total = L.order + rgx_align_up(L.order_words * sizeof(uint32_t), 256);
     return L;
@@ -2101,7 +2122,7 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
         march->max_prim_slice < 0 || !(march->dt_step > 0.0f) || ((uintptr_t)prims & 15u))
         return RGX_EINVAL;
     const MarchWs M = march_ws_layout(n, 0);
-    if (!march_ws || march_ws_bytes < M.order || ((uintptr_t)march_ws & 255u)) return RGX_EWORKSPACE;
+    if (!march_ws || march_ws_bytes < M.faults || ((uintptr_t)march_ws & 255u)) return RGX_EWORKSPACE;
     const WsLayout L = rgx_ws_layout(n);
     const char *w = (const char *)ws;
     P.cam = *cam;
@@ -2129,6 +2150,7 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     const size_t order_words = (size_t)8 * g.per_xcd * g.bw * g.bh;
     P.tile_order = M.order + order_words * sizeof(uint32_t) <= march_ws_bytes ? (uint32_t *)((char *)march_ws + M.order) : nullptr;
     P.use_tile_order = 0;
+    P.faults = M.order <= march_ws_bytes ? (uint32_t *)((char *)march_ws + M.faults) : nullptr;
     P.sum_pool = nullptr;
     P.sum_next = nullptr;
     P.sum_slots = 0;
@@ -2175,6 +2197,7 @@ extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const Rgx
                                  float *ray_colors, void *march_ws, size_t march_ws_bytes, void *records, size_t records_bytes,
                                  RgxStats *stats, void *stream)
 {
+    const DeviceScope on_device(ws);
     MarchParams P;
     int rc = fill_params(P, ws, cam, march, prims, n, march_ws, march_ws_bytes, stats);
     if (rc) return rc;
@@ -2183,8 +2206,8 @@ extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const Rgx
     if (rc) return rc;
     P.ray_colors = ray_colors;
     void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
+    if (P.sum_pool || P.faults) hipLaunchKernelGGL(k_clear2, dim3(1), dim3(64), 0, (hipStream_t)stream, (float4 *)P.sum_next, (float4 *)P.faults);
     if (P.records) {
-        if (P.sum_pool) hipLaunchKernelGGL(k_zero4, dim3(1), dim3(64), 0, (hipStream_t)stream, (float4 *)P.sum_next, (int64_t)1);
         if (stats) hipLaunchKernelGGL((k_march_fwd<true, false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
         else hipLaunchKernelGGL((k_march_fwd<true, false, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     } else {
@@ -2199,6 +2222,7 @@ extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const Rgx
 extern "C" int rgx_march_viewer(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
                                 uint8_t *frame, float *depth, void *march_ws, size_t march_ws_bytes, RgxStats *stats, void *stream)
 {
+    const DeviceScope on_device(ws);
     MarchParams P;
     const int rc = fill_params(P, ws, cam, march, prims, n, march_ws, march_ws_bytes, stats);
     if (rc != RGX_OK) return rc;
@@ -2206,6 +2230,7 @@ extern "C" int rgx_march_viewer(const void *ws, const RgxCamera *cam, const RgxM
     P.frame = frame;
     P.depth = depth;
     void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
+    if (P.faults) hipLaunchKernelGGL(k_clear2, dim3(1), dim3(64), 0, (hipStream_t)stream, (float4 *)nullptr, (float4 *)P.faults);
     if (stats) hipLaunchKernelGGL((k_march_fwd<false, true, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     else hipLaunchKernelGGL((k_march_fwd<false, true, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     rgx_span_end(span, (hipStream_t)stream);
@@ -2218,6 +2243,7 @@ extern "C" int rgx_march_backward(const void *ws, const RgxCamera *cam, const Rg
                                   float *dscale, float *dquat, void *march_ws, size_t march_ws_bytes, const void *records,
                                   size_t records_bytes, RgxStats *stats, void *stream)
 {
+    const DeviceScope on_device(ws);
     MarchParams P;
     int rc = fill_params(P, ws, cam, march, prims, n, march_ws, march_ws_bytes, stats);
     if (rc) return rc;
@@ -2257,6 +2283,21 @@ extern "C" int rgx_march_backward(const void *ws, const RgxCamera *cam, const Rg
     return RGX_OK;
 }
 
+extern "C" int rgx_march_faults(const void *march_ws, size_t march_ws_bytes, int64_t n, uint64_t *host_out2, void *stream)
+{
+    if (!march_ws || n < 0 || !host_out2) return RGX_EINVAL;
+    const DeviceScope on_device(march_ws);
+    const MarchWs M = march_ws_layout(n, 0);
+    host_out2[0] = host_out2[1] = 0;
+    if (M.order > march_ws_bytes) return RGX_OK; // no room for the counters: none kept
+    uint32_t words[2] = {0, 0};
+    RGX_HIP(hipMemcpyAsync(words, (const char *)march_ws + M.faults, sizeof words, hipMemcpyDeviceToHost, (hipStream_t)stream));
+    RGX_HIP(hipStreamSynchronize((hipStream_t)stream));
+    host_out2[0] = words[0];
+    host_out2[1] = words[1];
+    return RGX_OK;
+}
+
 static int hook_params(MarchParams &P, const void *ws, const float *prims, int64_t n_prims)
 {
     if (!ws || n_prims < 0 || (n_prims > 0 && !prims)) return RGX_EINVAL;
@@ -2275,6 +2316,7 @@ static int hook_params(MarchParams &P, const void *ws, const float *prims, int64
 extern "C" int rgx_first_hit(const void *ws, const float *prims, int64_t n_prims, const float *eye, int64_t n,
                              const float *dirs, const float *tlo, const float *thi, float *out_t, void *stream)
 {
+    const DeviceScope on_device(ws);
     MarchParams P;
     const int rc = hook_params(P, ws, prims, n_prims);
     if (rc) return rc;
@@ -2290,6 +2332,7 @@ extern "C" int rgx_trace_segments(const void *ws, const float *prims, int64_t n_
                                   const float *dirs, const float *tlo, const float *thi, int32_t cap, int32_t *counts,
                                   int32_t *ids, void *stream)
 {
+    const DeviceScope on_device(ws);
     MarchParams P;
     const int rc = hook_params(P, ws, prims, n_prims);
     if (rc) return rc;
@@ -2302,8 +2345,9 @@ extern "C" int rgx_trace_segments(const void *ws, const float *prims, int64_t n_
 }
 
 extern "C" int rgx_collect_tiles(const void *ws, const RgxCamera *cam, const float *prims, int64_t n_prims, const float *tlo,
-                                 const float *thi, int32_t cap, int32_t *counts, int32_t *ids, void *stream)
+                                 const float *thi, int32_t cap, int32_t *counts, int32_t *ids, int32_t uncounted, void *stream)
 {
+    const DeviceScope on_device(ws);
     MarchParams P;
     const int rc = hook_params(P, ws, prims, n_prims);
     if (rc) return rc;
@@ -2311,7 +2355,8 @@ extern "C" int rgx_collect_tiles(const void *ws, const RgxCamera *cam, const flo
     P.cam = *cam;
     P.tiles_x = (cam->width + 7) / 8;
     P.tiles_y = (cam->height + 7) / 8;
-    hipLaunchKernelGGL(k_collect_tiles, march_grid(P), dim3(64), 0, (hipStream_t)stream, P, tlo, thi, (int)cap, counts, ids);
+    if (uncounted) hipLaunchKernelGGL(k_collect_tiles<false>, march_grid(P), dim3(64), 0, (hipStream_t)stream, P, tlo, thi, (int)cap, counts, ids);
+    else hipLaunchKernelGGL(k_collect_tiles<true>, march_grid(P), dim3(64), 0, (hipStream_t)stream, P, tlo, thi, (int)cap, counts, ids);
     RGX_LAUNCH_CHECK();
     return RGX_OK;
 }
@@ -2333,6 +2378,7 @@ __global__ __launch_bounds__(256) void k_check_plain_arith(const float *__restri
 
 extern "C" int rgx_check_plain_arith(const float *a, const float *b, int64_t n, uint32_t *bad, void *stream)
 {
+    const DeviceScope on_device(a);
     if (n < 0 || (n > 0 && (!a || !b)) || !bad) return RGX_EINVAL;
     if (n > 0) hipLaunchKernelGGL(k_check_plain_arith, grid_for(n, 256), dim3(256), 0, (hipStream_t)stream, a, b, n, bad);
     RGX_LAUNCH_CHECK();

@@ -171,6 +171,7 @@ static int sh_forward_launch(const float *eye, const float *pos, const float *sh
                              const float *axis, int32_t g, int32_t degree, int32_t gs, int32_t ks, int64_t n, float *rgb,
                              void *stream)
 {
+    const DeviceScope on_device(pos);
     if (!eye || n < 0 || degree < 0 || degree > 3 || g < 0 || gs < g || ks < (degree + 1) * (degree + 1) ||
         (n > 0 && (!pos || !sh || !rgb)) || (g > 0 && n > 0 && (!sg || !sharp || !axis)))
         return RGX_EINVAL;
@@ -207,6 +208,7 @@ extern "C" int rgx_sh_backward(const float *eye, const float *pos, const float *
                                const float *axis, int32_t g, int32_t degree, int64_t n, const float *drgb, float *dsh,
                                float *dpos, float *dsg, float *dsharp, float *daxis, void *stream)
 {
+    const DeviceScope on_device(pos);
     if (!eye || n < 0 || degree < 0 || degree > 3 || g < 0 || (n > 0 && (!pos || !sh || !drgb || !dsh || !dpos)) ||
         (g > 0 && n > 0 && (!sg || !sharp || !axis || !dsg || !dsharp || !daxis)))
         return RGX_EINVAL;
@@ -234,6 +236,7 @@ extern "C" int rgx_pack_prims(const void *ws, const float *eye, const float *pos
                               const float *dens, const float *rgb, int64_t n, float sigma_threshold, float *prims,
                               void *stream)
 {
+    const DeviceScope on_device(prims);
     if (!eye || n < 0 || (n > 0 && (!pos || !scale || !quat || !dens || !rgb || !prims)) || ((uintptr_t)prims & 15u))
         return RGX_EINVAL;
     if (n == 0) return RGX_OK;

@@ -16,17 +16,24 @@ from . import _lib as L
 SIGMA_THRESHOLD = 0.1            # cuda_train/forward/gaussians_aabb.h:5
 TRANSMITTANCE_EPSILON = 1e-3     # cuda_train/forward/gaussians_aabb.h:4
 
-_scratch = {}
+_scratch = {}          # (key, device, stream handle) -> byte tensor, most recently used last
+_SCRATCH_STREAMS = 8   # scratch sets kept per key and device: one per stream in use; older ones are dropped
 
 
 def _workspace(key, nbytes, device):
     """Cached byte tensor (grown, never shrunk) -- keeps the hot path free of allocations.  One per
-    stream: views rendered on different streams run concurrently and must not share scratch memory."""
-    slot = (key, device, torch.cuda.current_stream(device).cuda_stream)
-    t = _scratch.get(slot)
+    stream: views rendered on different streams run concurrently and must not share scratch memory.
+    A loop that keeps creating streams does not accumulate them: per key and device only the
+    ``_SCRATCH_STREAMS`` most recently used streams keep their tensor (a dropped tensor's memory goes
+    back to torch's allocator, which keeps it alive for work already queued on its stream)."""
+    slot = (key, str(device), torch.cuda.current_stream(device).cuda_stream)
+    t = _scratch.pop(slot, None)
     if t is None or t.numel() < nbytes:
         t = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
-        _scratch[slot] = t
+    _scratch[slot] = t          # re-inserted: dicts keep insertion order, so this is now the newest
+    mine = [k for k in _scratch if k[0] == key and k[1] == str(device)]
+    for k in mine[:-_SCRATCH_STREAMS]:
+        del _scratch[k]
     return t
 
 
@@ -122,10 +129,9 @@ def create_context(log=None):
 
 
 def create_module(ctx, pipeline_opts, stage, debug_level=None, opt_level=None):
+    """optix_utils.py:148-178.  "gui" stands for the viewer's kernels (``march_viewer``, ``sh_viewer``)."""
     if stage not in ("forward", "backward", "test", "gui"):
         raise ValueError("stage must be 'forward', 'backward', 'test' or 'gui'")
-    if stage == "gui":
-        raise NotImplementedError("the GUI kernel variant is not part of this library")
     L.lib()  # make a missing library surface here, like a failed module compile would
     return _Handle("module", stage=stage)
 
@@ -357,11 +363,25 @@ def trace_segments(gas, prims, eye, dirs, tlo, thi, cap):
     return counts, ids
 
 
-def collect_tiles(gas, cam, prims, tlo, thi, cap):
-    """Hit lists of per-pixel segments through the tile-cooperative collect (test hook)."""
+def collect_tiles(gas, cam, prims, tlo, thi, cap, uncounted=False):
+    """Hit lists of per-pixel segments through the tile-cooperative collect (test hook).  ``uncounted``:
+    the filter as the kernels launched without a statistics block compile it (with its early exit)."""
     n_rays = cam.width * cam.height
     counts = torch.zeros(n_rays, dtype=torch.int32, device=prims.device)
     ids = torch.full((n_rays, cap), -1, dtype=torch.int32, device=prims.device)
     L.check(L.lib().rgx_collect_tiles(L.ptr(gas.ws), C.byref(cam), L.ptr(prims), C.c_int64(prims.shape[0]), L.ptr(tlo),
-                                      L.ptr(thi), C.c_int32(cap), L.ptr(counts), L.ptr(ids), L.stream(prims.device)))
+                                      L.ptr(thi), C.c_int32(cap), L.ptr(counts), L.ptr(ids), C.c_int32(int(bool(uncounted))),
+                                      L.stream(prims.device)))
     return counts, ids
+
+
+def march_faults(n, device, ws=None):
+    """(replays that lost their record, sweeps that dropped nodes) counted by the launches since the last
+    forward on this stream's march workspace; waits for the stream."""
+    if ws is None:
+        ws = _scratch.get(("march", str(device), torch.cuda.current_stream(device).cuda_stream))
+        if ws is None:
+            return 0, 0
+    out = (C.c_uint64 * 2)()
+    L.check(L.lib().rgx_march_faults(L.ptr(ws), C.c_size_t(ws.numel()), C.c_int64(n), out, L.stream(device)))
+    return int(out[0]), int(out[1])

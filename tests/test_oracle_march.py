@@ -123,6 +123,153 @@ def _f64_march_image(sc, cam, dt, ids, eps=1e-3):
     return out
 
 
+def _f64_march_adaptive(sc, cam, dt0, ids, eps=1e-3, dynamic=True):
+    """Independent float64 march with the step rule of gaussians_aabb.cu:266-273 recomputed from its OWN
+    transmittance and position: dt = min(max(t / 1024, dt0) * T^(-1/3), 4 dt0), slab = 32 dt; every
+    sample's Mahalanobis distance evaluated directly.  Returns the image, per ray the blended slabs
+    [(t, dt, sorted ids)], and per ray a margin: the smallest relative distance between a decision the
+    march took (a Gaussian's entry or exit against a slab boundary, T against eps) and its flipping
+    point.  A float32 march of the same rule can only differ in its slab sequence on rays whose margin
+    is of the order of float32 rounding."""
+    eye = cam.camera_center.double().numpy()
+    dirs = f64ref.ray_dirs_pinhole(cam, ids)
+    pos, scale, quat, dens = (sc[k].astype(np.float64) for k in ("positions", "scales", "quaternions", "densities"))
+    rgb = 0.5 + 0.28209479177387814 * sc["color_features"][:, :, 0].astype(np.float64)
+    valid, t_in, t_out, closest2 = f64ref.ellipsoid_roots(eye, dirs, pos, scale, quat, dens)
+    near_graze = ((closest2 - (1 - 1e-7)).abs() < 1e-5).numpy()     # the predicate's disc > 1e-7 test
+    valid = (valid & (closest2 < 1 - 1e-7)).numpy()
+    t_in, t_out = t_in.numpy(), t_out.numpy()
+    R = f64ref.rot_from_quat(torch.tensor(quat)).numpy()
+    kk = 2 * np.log(dens / 0.1)
+    out = np.ones((len(ids), 3))
+    seqs, margins = [], []
+    for r in range(len(ids)):
+        cand = np.nonzero(valid[r] & (t_out[r] >= 0))[0]
+        seq, margin = [], np.inf
+        if near_graze[r].any():
+            margin = 0.0
+        if len(cand):
+            tb = max(t_in[r, cand].min(), 0.0)
+            tend = t_out[r, cand].max()
+            T, C = 1.0, np.zeros(3)
+            dt = dt0
+            while tb <= tend and T > eps:
+                margin = min(margin, abs(T - eps) / eps)
+                if dynamic:
+                    dt = min(max(tb / 1024.0, dt0) * T ** (-1.0 / 3.0), 4.0 * dt0)
+                L = 32 * dt
+                ci, co = t_in[r, cand], t_out[r, cand]
+                margin = min(margin, np.abs(ci - (tb + L)).min() / (tb + L), np.abs(co - tb).min() / tb)
+                hit = cand[(ci <= tb + L) & (co >= tb)]
+                if len(hit) == 0:
+                    nxt = cand[co >= tb + L]
+                    if len(nxt) == 0:
+                        break
+                    tb = max(t_in[r, nxt].min(), tb + L)
+                    continue
+                seq.append((tb, dt, np.sort(hit)))
+                t = tb + dt * (np.arange(32) + 0.5)
+                x = eye[None] + t[:, None] * dirs[r][None]
+                loc = np.einsum("hji,hsj->hsi", R[hit], x[None] - pos[hit][:, None]) / scale[hit][:, None]
+                power = (loc ** 2).sum(-1)
+                w = np.exp(-0.5 * power) * (power < kk[hit][:, None])
+                sig = (dens[hit][:, None] * w).sum(0)
+                col = ((dens[hit][:, None] * w)[:, :, None] * rgb[hit][:, None]).sum(0)
+                for base in (0, 16):
+                    if T <= eps:
+                        break
+                    if base:
+                        margin = min(margin, abs(T - eps) / eps)
+                    for i in range(base, base + 16):
+                        xx = sig[i] * dt
+                        ww = math.exp(-xx)
+                        C += T * dt * (1 - ww) / max(xx, 1e-6) * col[i]
+                        T *= ww
+                tb += L
+            margin = min(margin, abs(T - eps) / eps)
+            out[r] = C + T
+        seqs.append(seq)
+        margins.append(margin)
+    return out, seqs, np.array(margins)
+
+
+def test_adaptive_step_matches_independent_float64_march(orc):
+    """Pins the dynamic_sampling branch (gaussians_aabb.cu:266-273).  The float64 march above recomputes
+    every step from its own transmittance; on rays where none of its decisions sits within 1e-4 of
+    flipping, the oracle must have marched the same slabs -- same count, same (t, dt) to float32
+    accuracy, same hit sets -- and produced the same colour.  A cbrt for the rcbrt, a dropped
+    4 dt0 cap, a wrong 1024 or a step taken from the previous slab's T all change dt by far more."""
+    checked = 0
+    for seed, n, mult, res in ((3, 1500, 3.0, 20), (8, 4000, 2.0, 16)):
+        sc = scenes.scene_to_numpy(scenes.make_scene(2, n=n, sh_degree=0, seed=seed))
+        sc["scales"] = sc["scales"] * mult
+        cam = scenes.make_camera(2, 1, width=res, height=res)
+        ids = np.arange(res * res)
+        dt0 = 0.005
+        img, st, ctx = _render(orc, sc, cam, dt0, dynamic=True, cap=n)
+        want, seqs, margins = _f64_march_adaptive(sc, cam, dt0, ids)
+        robust = margins > 1e-4
+        assert robust.mean() > 0.8 and st["overflow_rays"] == 0
+        steps_seen = set()
+        for r in np.nonzero(robust)[0]:
+            slabs, _ = orc.march_trace(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], int(r))
+            got = [(tb, dt, np.sort(i)) for tb, dt, lo, hi, i in slabs if len(i)]
+            assert len(got) == len(seqs[r]), (seed, r, len(got), len(seqs[r]))
+            for (tb, dt, hit), (tb64, dt64, hit64) in zip(got, seqs[r]):
+                assert abs(tb - tb64) <= 2e-5 * tb64 and abs(dt - dt64) <= 2e-5 * dt64, (seed, r, tb, tb64, dt, dt64)
+                assert np.array_equal(hit, hit64), (seed, r)
+                steps_seen.add(round(dt64 / dt0, 2))
+            checked += len(got)
+        # the steps met span the rule's whole range: dt0 (T = 1 near the camera) up to the 4 dt0 cap
+        assert min(steps_seen) < 1.05 and max(steps_seen) == 4.0 and len(steps_seen) > 20
+        err = np.abs(img[ids] - want).max(1)[robust]
+        assert np.quantile(err, 0.98) < 2e-5 and err.max() < 6e-4     # one flipped cut-off sample costs <= 0.1 * 4 dt0 * |dc|
+    assert checked > 1500
+
+
+def test_adaptive_step_closed_forms_on_one_gaussian(orc):
+    """The step rule against what the mathematics fixes, on one isotropic Gaussian on the ray axis
+    (transmittance known in closed form through erf):
+    (i) the first slab has T = 1, so dt = max(t_enter / 1024, dt0) exactly -- the distance term alone,
+        on both sides of its max and up to where it alone reaches the cap;
+    (ii) further in, dt = dt_dist * T(t)^(-1/3) with the analytic T(t);
+    (iii) once T < 1/64 the step is the cap 4 dt0 exactly, until T < eps ends the ray."""
+    dt0, s = 0.005, 0.3
+    # (a tiny eps keeps the dense cases marching after T < 1/64, where the cap is the whole rule)
+    for rho, dist, eps in ((3.0, 4.0, 1e-3), (3.0, 12.0, 1e-3), (3.0, 40.0, 1e-3), (30.0, 4.0, 1e-9), (80.0, 9.0, 1e-9)):
+        k = math.sqrt(2 * math.log(rho / 0.1))
+        cam = _axis_camera(dist=dist)
+        img, st, ctx = _render(orc, _one_gaussian(rho, s, (0.2, 0.6, 0.9)), cam, dt0, dynamic=True, eps=eps)
+        slabs, _ = orc.march_trace(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], 4 * 9 + 4)
+        slabs = [sl for sl in slabs if len(sl[4])]
+        assert len(slabs) >= 2
+        t_enter = dist - k * s
+        assert abs(slabs[0][0] - t_enter) < 1e-4
+        # (i): float32 arithmetic of the rule with T = 1 (rcbrt(1) = 1)
+        first = min(max(np.float32(slabs[0][0]) / np.float32(1024.0), np.float32(dt0)), np.float32(4.0) * np.float32(dt0))
+        assert np.float32(slabs[0][1]) == first, (rho, dist, slabs[0][1], first)
+
+        def T_analytic(t):      # exp(-int_{t_enter}^{t} rho exp(-(u - dist)^2 / (2 s^2)) du)
+            a, b = (t_enter - dist) / (s * math.sqrt(2)), (min(t, dist + k * s) - dist) / (s * math.sqrt(2))
+            return math.exp(-rho * s * math.sqrt(math.pi / 2) * (math.erf(b) - math.erf(a)))
+
+        saturated = grew = 0
+        for tb, dt, lo, hi, _ in slabs[1:]:
+            T = T_analytic(tb)
+            want = min(max(tb / 1024.0, dt0) * T ** (-1.0 / 3.0), 4 * dt0)
+            # the oracle's T is a midpoint-rule product: O(dt^2) off the analytic one, plus the 0.1 density
+            # jump at the truncation boundary
+            assert abs(dt - want) <= 2e-3 * want, (rho, dist, tb, dt, want)
+            if T < 1.0 / 64.0 * 0.98:
+                assert np.float32(dt) == np.float32(4.0) * np.float32(dt0)      # (iii): the cap, exactly
+                saturated += 1
+            grew += dt > slabs[0][1] * 1.01
+        if rho >= 30.0:
+            assert saturated >= 1
+        if dist <= 12.0:
+            assert grew >= 1            # (ii): the step really grows with falling T
+
+
 def test_forward_matches_independent_float64_march(orc):
     sc = scenes.scene_to_numpy(scenes.make_scene(0, n=600, sh_degree=0, seed=21))
     sc["scales"] = sc["scales"] * 2.5

@@ -179,6 +179,14 @@ int rgx_march_forward(const void *ws, const RgxCamera *cam, const RgxMarch *marc
                       int64_t n, float *ray_colors, void *march_ws, size_t march_ws_bytes,
                       void *records, size_t records_bytes, RgxStats *stats, void *stream);
 
+/* Test hook: rgx_march_forward through the counting kernels, with the counters also kept per ray:
+ * ray_counts (W*H, 2) = slabs blended and the sum of their hit-list lengths (the per-ray share of
+ * RgxStats.slabs / hit_pairs).  Lets a test tell which rays marched the same slab sequence as a CPU
+ * evaluation when the adaptive step makes that depend on the last bit of cbrt / exp. */
+int rgx_march_forward_counts(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims,
+                             int64_t n, float *ray_colors, void *march_ws, size_t march_ws_bytes, void *records,
+                             size_t records_bytes, RgxStats *stats, uint32_t *ray_counts, void *stream);
+
 /* Replaces launch_pipeline_backward + reduce_temp_grads (optix_utils.py:325-500) and
  * cuda_train/backward/gaussians_aabb.cu: gradients of sum(dloss * ray_colors) with
  * respect to density (N), rgb (N,3), position (N,3), scale (N,3), quaternion (N,4),

@@ -76,6 +76,7 @@ struct MarchParams {
     uint32_t *sum_next;     // next free slot (bump counter in the record's pool header)
     int32_t sum_slots;      // slots in the pool
     uint32_t *faults;       // march workspace: [0] replays that lost their record, [1] sweeps that dropped nodes; or null
+    uint32_t *ray_counts;   // counting forward only: per ray, slabs blended and the sum of their hit-list lengths; or null
 };
 
 // Launch statistics (RgxStats).  Kernels launched without a statistics block carry none of it:
@@ -1664,6 +1665,13 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
             P.ray_colors[3 * ray + 2] = Cb + R.T * bg;
         }
     }
+    if constexpr (STATS) {
+        if (valid && P.ray_counts) {
+            const int64_t ray = (int64_t)py * P.cam.width + px;
+            P.ray_counts[2 * ray] = cn.slabs;
+            P.ray_counts[2 * ray + 1] = cn.hit_pairs;
+        }
+    }
     rec.finish(P);
     flush_stats(P.stats, cn);
 }
@@ -2151,6 +2159,7 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     P.tile_order = M.order + order_words * sizeof(uint32_t) <= march_ws_bytes ? (uint32_t *)((char *)march_ws + M.order) : nullptr;
     P.use_tile_order = 0;
     P.faults = M.order <= march_ws_bytes ? (uint32_t *)((char *)march_ws + M.faults) : nullptr;
+    P.ray_counts = nullptr;
     P.sum_pool = nullptr;
     P.sum_next = nullptr;
     P.sum_slots = 0;
@@ -2193,9 +2202,30 @@ static inline dim3 march_grid(const MarchParams &P)
     return dim3((unsigned)(8 * g.per_xcd * g.bw * g.bh));
 }
 
+static int march_forward_launch(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
+                                float *ray_colors, void *march_ws, size_t march_ws_bytes, void *records, size_t records_bytes,
+                                RgxStats *stats, uint32_t *ray_counts, void *stream);
+
 extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
                                  float *ray_colors, void *march_ws, size_t march_ws_bytes, void *records, size_t records_bytes,
                                  RgxStats *stats, void *stream)
+{
+    return march_forward_launch(ws, cam, march, prims, n, ray_colors, march_ws, march_ws_bytes, records, records_bytes, stats,
+                                nullptr, stream);
+}
+
+extern "C" int rgx_march_forward_counts(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
+                                        float *ray_colors, void *march_ws, size_t march_ws_bytes, void *records,
+                                        size_t records_bytes, RgxStats *stats, uint32_t *ray_counts, void *stream)
+{
+    if (!ray_counts) return RGX_EINVAL;
+    return march_forward_launch(ws, cam, march, prims, n, ray_colors, march_ws, march_ws_bytes, records, records_bytes, stats,
+                                ray_counts, stream);
+}
+
+static int march_forward_launch(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
+                                float *ray_colors, void *march_ws, size_t march_ws_bytes, void *records, size_t records_bytes,
+                                RgxStats *stats, uint32_t *ray_counts, void *stream)
 {
     const DeviceScope on_device(ws);
     MarchParams P;
@@ -2205,13 +2235,15 @@ extern "C" int rgx_march_forward(const void *ws, const RgxCamera *cam, const Rgx
     rc = attach_records(P, records, records_bytes);
     if (rc) return rc;
     P.ray_colors = ray_colors;
+    P.ray_counts = ray_counts;
+    const bool counting = stats != nullptr || ray_counts != nullptr;
     void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
     if (P.sum_pool || P.faults) hipLaunchKernelGGL(k_clear2, dim3(1), dim3(64), 0, (hipStream_t)stream, (float4 *)P.sum_next, (float4 *)P.faults);
     if (P.records) {
-        if (stats) hipLaunchKernelGGL((k_march_fwd<true, false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+        if (counting) hipLaunchKernelGGL((k_march_fwd<true, false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
         else hipLaunchKernelGGL((k_march_fwd<true, false, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     } else {
-        if (stats) hipLaunchKernelGGL((k_march_fwd<false, false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+        if (counting) hipLaunchKernelGGL((k_march_fwd<false, false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
         else hipLaunchKernelGGL((k_march_fwd<false, false, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     }
     rgx_span_end(span, (hipStream_t)stream);

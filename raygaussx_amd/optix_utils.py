@@ -235,12 +235,21 @@ def new_records(cam, device, tile_words=REC_TILE_WORDS, budget_bytes=None):
 
 
 def march_forward(gas, cam, prims, dt_step, dynamic_sampling, max_prim_slice, white_background,
-                  t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None):
+                  t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None, ray_counts=False):
+    """``ray_counts=True`` (test hook): also returns an (n_rays, 2) int32 tensor, per ray the slabs blended and
+    the sum of their hit-list lengths."""
     n, dev = prims.shape[0], prims.device
     n_rays = cam.width * cam.height
     m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), int(bool(white_background)), t_eps)
     ws = _march_ws(n, n_rays, max_prim_slice, dev)
     ray_colors = torch.empty(n_rays, 3, dtype=torch.float32, device=dev)
+    if ray_counts:
+        counts = torch.zeros(n_rays, 2, dtype=torch.int32, device=dev)
+        L.check(L.lib().rgx_march_forward_counts(L.ptr(gas.ws), C.byref(cam), C.byref(m), L.ptr(prims), C.c_int64(n),
+                                                 L.ptr(ray_colors), L.ptr(ws), C.c_size_t(ws.numel()), L.ptr(records),
+                                                 C.c_size_t(0 if records is None else records.numel()), L.ptr(stats),
+                                                 L.ptr(counts), L.stream(dev)))
+        return ray_colors, counts
     L.check(L.lib().rgx_march_forward(L.ptr(gas.ws), C.byref(cam), C.byref(m), L.ptr(prims), C.c_int64(n),
                                       L.ptr(ray_colors), L.ptr(ws), C.c_size_t(ws.numel()), L.ptr(records),
                                       C.c_size_t(0 if records is None else records.numel()), L.ptr(stats),
@@ -373,6 +382,49 @@ def collect_tiles(gas, cam, prims, tlo, thi, cap, uncounted=False):
                                       L.ptr(thi), C.c_int32(cap), L.ptr(counts), L.ptr(ids), C.c_int32(int(bool(uncounted))),
                                       L.stream(prims.device)))
     return counts, ids
+
+
+_fault_watch = {}    # (device, stream handle) -> [pinned int32 tensor, event, pending]
+FAULTS_SEEN = {"replay_lost": 0, "sweep_dropped": 0}   # totals of what the lazy checks below have read so far
+
+
+def _watch_faults(ws, n, device):
+    """After a backward: queue a 16-byte copy of the workspace's fault counters to pinned host memory.
+    Nothing waits for it; ``_check_faults`` looks at it when the same stream next starts a forward."""
+    off = (max(int(n), 1) * 64 + 255) // 256 * 256
+    if ws.numel() < off + 256:
+        return
+    key = (str(device), torch.cuda.current_stream(device).cuda_stream)
+    w = _fault_watch.get(key)
+    if w is None:
+        w = _fault_watch[key] = [torch.zeros(4, dtype=torch.int32).pin_memory(), torch.cuda.Event(), False]
+        if len(_fault_watch) > 4 * _SCRATCH_STREAMS:
+            del _fault_watch[next(iter(_fault_watch))]
+    if w[2] and not w[1].query():
+        return                              # the previous copy is still in flight: keep its buffer untouched
+    w[0].copy_(ws[off:off + 16].view(torch.int32), non_blocking=True)
+    w[1].record(torch.cuda.current_stream(device))
+    w[2] = True
+
+
+def _check_faults(device):
+    """Reads the counters a finished ``_watch_faults`` copy brought back.  A sweep that dropped tree nodes
+    lost hits (wrong image and gradients): RgxError.  A replay that lost its record gave that tile the
+    gradient of the iterations replayed so far (a difference at the transmittance floor): a warning."""
+    w = _fault_watch.get((str(device), torch.cuda.current_stream(device).cuda_stream))
+    if w is None or not w[2] or not w[1].query():
+        return
+    w[2] = False
+    lost, dropped = int(w[0][0]), int(w[0][1])
+    FAULTS_SEEN["replay_lost"] += lost
+    FAULTS_SEEN["sweep_dropped"] += dropped
+    if dropped:
+        raise L.RgxError(f"librgx: {dropped} sweeps of an earlier launch dropped tree nodes (node stack full): "
+                         "hits were lost, its image and gradients are wrong")
+    if lost:
+        import warnings
+        warnings.warn(f"librgx: {lost} tiles of an earlier backward did not consume their hit-list record exactly; "
+                      "their gradients stop at the last iteration replayed", RuntimeWarning, stacklevel=3)
 
 
 def march_faults(n, device, ws=None):

@@ -107,6 +107,7 @@ class RenderOptixFunction(torch.autograd.Function):
         sph_gauss_features, bandwidth_sharpness, lobe_axis = (
             L.f32(t.detach()) for t in (sph_gauss_features, bandwidth_sharpness, lobe_axis))
         n, dev = positions.shape[0], positions.device
+        u_ox._check_faults(dev)     # what the previous backward on this stream reported, if it has finished
         # render_optix.py:109-117: boxes + acceleration structure (rebuilt unless settings.update)
         gas = settings.gas
         stale = gas is None or not isinstance(gas, u_ox.AccelerationStructure) or gas.n != n or gas.device != dev
@@ -146,6 +147,9 @@ class RenderOptixFunction(torch.autograd.Function):
                 settings.dynamic_sampling, settings.max_prim_slice, settings.white_background, settings.t_eps,
                 settings.stats, ctx.records)
             ctx.records = None
+            ws = u_ox._scratch.get(("march", str(positions.device), torch.cuda.current_stream(positions.device).cuda_stream))
+            if ws is not None:
+                u_ox._watch_faults(ws, positions.shape[0], positions.device)
             sh_grad, dpos_dir, dsg, dsharp, daxis = compute_sh_grad(
                 ctx.cam.eye, positions, color_features, sph_gauss_features, bandwidth_sharpness, lobe_axis,
                 settings.num_sph_gauss, ctx.order_sh, rgb_grad)

@@ -36,6 +36,7 @@ extern "C" {
 #define RGX_EINVAL -1     /* bad argument (null pointer, negative size, unsupported degree ...) */
 #define RGX_EWORKSPACE -2 /* workspace too small or misaligned */
 #define RGX_EHIP -3       /* a HIP runtime call failed; see rgx_last_hip_error() */
+#define RGX_ELIMIT -4     /* a size beyond the fixed limits of rgx_march_backward_noalloc() */
 
 /* Launch constants of one view.  Mirrors the camera part of `Params`
  * (optix_raycasting/cuda_train/forward/gaussians_aabb.h:14-44) as filled at
@@ -197,6 +198,23 @@ int rgx_march_backward(const void *ws, const RgxCamera *cam, const RgxMarch *mar
                        float *drgb, float *dpos, float *dscale, float *dquat, void *march_ws,
                        size_t march_ws_bytes, const void *records, size_t records_bytes,
                        RgxStats *stats, void *stream);
+
+/* rgx_march_backward for callers that cannot allocate device memory or bring a workspace: code
+ * under HIP graph capture, tight serving / fine-tuning loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference.  Same arguments and results as rgx_march_backward
+ * without march_ws: the gradient block and the tile order live in a file-scope device array of
+ * the library instead (RGX_NOALLOC_SCRATCH_BYTES, about 64.3 MiB, held by every GPU the library
+ * runs on until the process ends).  Limits: n <= RGX_NOALLOC_MAX_GAUSSIANS and width * height <=
+ * RGX_NOALLOC_MAX_RAYS, else RGX_ELIMIT.  The call allocates nothing, frees nothing and does not
+ * synchronise; it clears the part of the array it uses with a kernel.  All calls on one GPU share
+ * that GPU's array: calls that overlap on one GPU (two streams, two threads) race -- order them. */
+#define RGX_NOALLOC_MAX_GAUSSIANS (1 << 20)
+#define RGX_NOALLOC_MAX_RAYS (1 << 22)
+#define RGX_NOALLOC_SCRATCH_BYTES 67444992 /* 64 bytes per Gaussian + 256 + 4 bytes per 8x8 tile * 5/4 + 8192 */
+int rgx_march_backward_noalloc(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims,
+                               int64_t n, const float *ray_colors, const float *dloss, float *ddens,
+                               float *drgb, float *dpos, float *dscale, float *dquat, const void *records,
+                               size_t records_bytes, RgxStats *stats, void *stream);
 
 /* Launch faults that do not stop a launch, counted in the march workspace (always, with or without a
  * statistics block) and read back here; synchronous, waits for `stream`.  host_out[0]: tiles whose

@@ -38,6 +38,7 @@ extern "C" const char *rgx_strerror(int code)
     case RGX_EINVAL: return "invalid argument";
     case RGX_EWORKSPACE: return "workspace too small or misaligned";
     case RGX_EHIP: return "HIP runtime error (see rgx_last_hip_error)";
+    case RGX_ELIMIT: return "size beyond the limits of the allocation-free entry point";
     default: return "unknown error";
     }
 }

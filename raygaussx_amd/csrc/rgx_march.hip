@@ -23,6 +23,7 @@
 // The per-lane skip-link queries below serve the segment test hooks (arbitrary rays).
 #include "rgx_device.h"
 
+#include <mutex>
 #include <type_traits>
 
 #ifndef RGX_QCAP
@@ -2270,12 +2271,76 @@ extern "C" int rgx_march_viewer(const void *ws, const RgxCamera *cam, const RgxM
     return RGX_OK;
 }
 
+// timed: record the event-timed spans (they may create events; the allocation-free entry point goes without)
+static int march_backward_launch(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
+                                 const float *ray_colors, const float *dloss, float *ddens, float *drgb, float *dpos,
+                                 float *dscale, float *dquat, void *march_ws, size_t march_ws_bytes, const void *records,
+                                 size_t records_bytes, RgxStats *stats, void *stream, bool timed);
+
 extern "C" int rgx_march_backward(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
                                   const float *ray_colors, const float *dloss, float *ddens, float *drgb, float *dpos,
                                   float *dscale, float *dquat, void *march_ws, size_t march_ws_bytes, const void *records,
                                   size_t records_bytes, RgxStats *stats, void *stream)
 {
     const DeviceScope on_device(ws);
+    return march_backward_launch(ws, cam, march, prims, n, ray_colors, dloss, ddens, drgb, dpos, dscale, dquat, march_ws,
+                                 march_ws_bytes, records, records_bytes, stats, stream, true);
+}
+
+// ---------------------------------------------------------------------------
+// rgx_march_backward_noalloc: the backward whose scratch memory -- gradient block, fault counters,
+// tile order: a march workspace for RGX_NOALLOC_MAX_GAUSSIANS Gaussians and RGX_NOALLOC_MAX_RAYS
+// rays -- is a file-scope device array instead of a buffer of the caller's.  Every GPU the library
+// runs on holds its own copy of the array, at its own address, until the process ends.  `scratch`
+// is the host-side stand-in of that array, not a device address: the device address is asked for
+// once per device (with that device current) and kept, and only that address goes to kernels.
+static __device__ __align__(256) unsigned char scratch[RGX_NOALLOC_SCRATCH_BYTES];
+
+#define RGX_NOALLOC_MAX_DEVICES 64
+static std::mutex g_scratch_mu;
+static void *g_scratch_ptr[RGX_NOALLOC_MAX_DEVICES]; // per device: the device address of its `scratch`, or null
+
+// The current device's copy of the array.
+static int noalloc_scratch(void **out)
+{
+    int dev = -1;
+    RGX_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= RGX_NOALLOC_MAX_DEVICES) return RGX_ELIMIT;
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        RGX_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return RGX_EHIP;
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return RGX_OK;
+}
+
+extern "C" int rgx_march_backward_noalloc(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims,
+                                          int64_t n, const float *ray_colors, const float *dloss, float *ddens, float *drgb,
+                                          float *dpos, float *dscale, float *dquat, const void *records, size_t records_bytes,
+                                          RgxStats *stats, void *stream)
+{
+    static_assert(RGX_NOALLOC_SCRATCH_BYTES % 256 == 0, "the array is a 256-byte aligned march workspace");
+    if (!ws || !cam || n < 0 || cam->width <= 0 || cam->height <= 0) return RGX_EINVAL;
+    if (n > RGX_NOALLOC_MAX_GAUSSIANS || (int64_t)cam->width * cam->height > RGX_NOALLOC_MAX_RAYS) return RGX_ELIMIT;
+    if (march_ws_layout(RGX_NOALLOC_MAX_GAUSSIANS, RGX_NOALLOC_MAX_RAYS).total != RGX_NOALLOC_SCRATCH_BYTES) return RGX_EWORKSPACE;
+    const DeviceScope on_device(ws);
+    void *scr = nullptr;
+    const int rc = noalloc_scratch(&scr);
+    if (rc) return rc;
+    // the launch clears what it reads of the array with a kernel (the gradient block of these n Gaussians; the tile
+    // order is rewritten in full before use), so the previous call's contents do not matter
+    return march_backward_launch(ws, cam, march, prims, n, ray_colors, dloss, ddens, drgb, dpos, dscale, dquat, scr,
+                                 RGX_NOALLOC_SCRATCH_BYTES, records, records_bytes, stats, stream, false);
+}
+
+static int march_backward_launch(const void *ws, const RgxCamera *cam, const RgxMarch *march, const float *prims, int64_t n,
+                                 const float *ray_colors, const float *dloss, float *ddens, float *drgb, float *dpos,
+                                 float *dscale, float *dquat, void *march_ws, size_t march_ws_bytes, const void *records,
+                                 size_t records_bytes, RgxStats *stats, void *stream, bool timed)
+{
     MarchParams P;
     int rc = fill_params(P, ws, cam, march, prims, n, march_ws, march_ws_bytes, stats);
     if (rc) return rc;
@@ -2287,7 +2352,7 @@ extern "C" int rgx_march_backward(const void *ws, const RgxCamera *cam, const Rg
     P.dloss = dloss;
     hipStream_t s = (hipStream_t)stream;
     hipLaunchKernelGGL(k_zero4, grid_for(4 * n, 256), dim3(256), 0, s, (float4 *)P.gbuf, 4 * n);
-    void *span = rgx_span_begin(RGX_T_MARCH_BWD, s);
+    void *span = timed ? rgx_span_begin(RGX_T_MARCH_BWD, s) : nullptr;
     if (P.records) {
         // tiles with a complete record replay it; the few whose record overflowed are recomputed
         if (P.tile_order) {
@@ -2307,7 +2372,7 @@ extern "C" int rgx_march_backward(const void *ws, const RgxCamera *cam, const Rg
     if (stats) hipLaunchKernelGGL(k_march_bwd<true>, march_grid(P), dim3(64), 0, s, P);
     else hipLaunchKernelGGL(k_march_bwd<false>, march_grid(P), dim3(64), 0, s, P);
     rgx_span_end(span, s);
-    span = rgx_span_begin(RGX_T_UNPERMUTE, s);
+    span = timed ? rgx_span_begin(RGX_T_UNPERMUTE, s) : nullptr;
     hipLaunchKernelGGL(k_unpermute_grads, grid_for(n, 256), dim3(256), 0, s, (const float4 *)P.gbuf, P.order, n, ddens, drgb,
                        dpos, dscale, dquat);
     rgx_span_end(span, s);

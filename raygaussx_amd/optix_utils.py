@@ -285,16 +285,16 @@ def sh_viewer(camera_center, positions, sh, sph_gauss_features, bandwidth_sharpn
 
 
 def march_backward(gas, cam, prims, ray_colors, dloss, dt_step, dynamic_sampling, max_prim_slice,
-                   white_background=True, t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None):
+                   white_background=True, t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None, out=None):
+    """``out``: five preallocated gradient tensors (density, rgb, position, scale, quaternion) to write into."""
     n, dev = prims.shape[0], prims.device
     n_rays = cam.width * cam.height
     m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), int(bool(white_background)), t_eps)
     ws = _march_ws(n, n_rays, max_prim_slice, dev)
-    ddens = torch.empty(n, dtype=torch.float32, device=dev)
-    drgb = torch.empty(n, 3, dtype=torch.float32, device=dev)
-    dpos = torch.empty(n, 3, dtype=torch.float32, device=dev)
-    dscale = torch.empty(n, 3, dtype=torch.float32, device=dev)
-    dquat = torch.empty(n, 4, dtype=torch.float32, device=dev)
+    ddens, drgb, dpos, dscale, dquat = out if out is not None else (
+        torch.empty(n, dtype=torch.float32, device=dev), torch.empty(n, 3, dtype=torch.float32, device=dev),
+        torch.empty(n, 3, dtype=torch.float32, device=dev), torch.empty(n, 3, dtype=torch.float32, device=dev),
+        torch.empty(n, 4, dtype=torch.float32, device=dev))
     L.check(L.lib().rgx_march_backward(L.ptr(gas.ws), C.byref(cam), C.byref(m), L.ptr(prims), C.c_int64(n),
                                        L.ptr(ray_colors), L.ptr(dloss), L.ptr(ddens), L.ptr(drgb), L.ptr(dpos),
                                        L.ptr(dscale), L.ptr(dquat), L.ptr(ws), C.c_size_t(ws.numel()),

@@ -15,6 +15,11 @@ upper-hemisphere orbit per step.  Inputs are resident in HBM before the timed re
 Prints ONE JSON line.  ``roofline`` prices the dominant kernel (the backward march) with its
 algorithmic bytes (64+56 B per ray-slab-hit + 24 B per ray) over its own HIP-event time;
 ``cpu_baseline`` times the CPU oracle on a bounded ray sample of the same workload.
+``fwd_fps_c3`` is the other half of the headline metric, measured in the same run: frames per second
+of the forward-only render of the 3 M-Gaussian scene at 1920x1080 along its orbit, tree built once,
+with a roofline of its own.  ``hbm_measured`` is the bandwidth a plain 1 GiB device-to-device copy
+reaches on this GPU (read + written bytes), the practical ceiling beside the 8 TB/s peak;
+``memory`` reports the peak device memory of the run and the record's allocated and used bytes.
 Beside the contract's keys: ``atomics`` (the gradient scatter's atomic adds per backward launch,
 counted by the kernels, over the launch's time) and ``views_in_flight`` (the same steps timed once
 more with two views in flight on two streams, as a loop that accumulates gradients over several
@@ -39,13 +44,23 @@ from raygaussx_amd.render_optix import RenderOptixFunction, default_settings  # 
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this
-# script scaled by a 1 GiB copy (--calibrate-copy); the counter readings are kept in
-# profiles/march_kernels_c4_1M_800x800.md.  Workloads without a measurement report null.
-MEASURED_TRAFFIC_BYTES = {
-    ("c4_1M_800x800", "march_backward"): 17.3e9,   # k_march_bwd_replay_sums<false>: 14.7 GB read (14.0 the sample sums), 2.6 GB written
-    ("c4_1M_800x800", "march_forward"): 15.6e9,    # k_march_fwd<true, false, false>: 1.3 GB read, 14.4 GB written (14.0 the sample sums)
-}
+PROFILES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
+
+
+def stored_traffic(workload, kernel_key):
+    """HBM bytes per launch of a march kernel as a profiler run measured them: rocprofv3 --pmc FETCH_SIZE /
+    WRITE_SIZE of this script, scaled by the same counters' reading for a 1 GiB copy (--calibrate-copy).
+    The summary under profiles/ holds the figure in a line `traffic_bytes_per_launch <workload> <kernel key> <bytes>`;
+    this run does not measure it (counters need the profiler), so the JSON line names the file it came from.
+    None when there is no such line."""
+    import glob
+    import re
+    for path in sorted(glob.glob(os.path.join(PROFILES, "*.md"))):
+        for line in open(path):
+            m = re.match(r"\s*traffic_bytes_per_launch\s+(\S+)\s+(\S+)\s+([0-9.eE+]+)", line)
+            if m and m.group(1) == workload and m.group(2) == kernel_key:
+                return float(m.group(3)), os.path.relpath(path, os.path.dirname(PROFILES))
+    return None, None
 
 WORKLOADS = {
     # name: (scene config, n, width, height)
@@ -60,23 +75,107 @@ WORKLOADS = {
 
 
 def cpu_baseline(scene, cam, cfg, n_sample, threads, backward=True):
-    """Forward (+ backward) of the CPU oracle on a strided ray sample of the same view."""
+    """The same step on the host cores: the CPU oracle's forward (+ backward) march on a strided ray sample
+    of the same view, candidates culled by its bounding-volume tree over the Gaussians' boxes (same results
+    as its brute force, see tests/test_oracle_geometry.py).  Timed: tree build + march of the sample; the
+    per-Gaussian colour / packing / SH gradient passes run once per view whatever the sample and are left out."""
     from oracle import oracle as orc
     orc.build()
     orc.set_num_threads(threads)
     sc = scenes.scene_to_numpy(scene)
     n_rays = cam.image_width * cam.image_height
     ids = np.linspace(0, n_rays - 1, n_sample).astype(np.int64)
+    few = ids[:: max(1, n_sample // 64)]
+    _, _, ctx = orc.render_forward(sc, cam, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
+                                   t_eps=cfg["t_eps"], ray_ids=few[:1])      # boxes, colours, primitive records
     t0 = time.perf_counter()
-    img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
-                                      ray_ids=ids)
-    if backward:
-        dloss = np.full(img.shape, 1.0 / img.size, np.float32)
-        orc.render_backward(sc, ctx, img, dloss)
+    orc.cull_build(ctx["prims"])
+    t_build = time.perf_counter() - t0
+    try:
+        img, _ = orc.march_forward(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], ids)
+        if backward:
+            dloss = np.full(img.shape, 1.0 / img.size, np.float32)
+            orc.march_backward(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], img, dloss, ids)
+    finally:
+        orc.cull_free()
     dt = time.perf_counter() - t0
     return dict(value=round(n_sample / dt / 1e6, 6), unit="Mrays/s", cores=threads, kind="port",
-                sample=f"{n_sample} strided rays of camera 0, {'fwd+bwd' if backward else 'fwd'}, all {sc['positions'].shape[0]} Gaussians "
-                       f"(brute-force hit search), {dt:.1f} s")
+                sample=f"{n_sample} strided rays of camera 0, {'fwd+bwd' if backward else 'fwd'} march, all {sc['positions'].shape[0]} "
+                       f"Gaussians behind a CPU bounding-volume tree ({t_build:.2f} s to build, included), {dt:.1f} s")
+
+
+def copy_bandwidth(dev, reps=10):
+    """GB/s (bytes read + bytes written) of a 1 GiB device-to-device copy: what a plain streaming kernel
+    reaches on this GPU, the practical ceiling beside the published peak."""
+    src = torch.full((1 << 28,), 1.0, dtype=torch.float32, device=dev)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        dst.copy_(src)
+    b.record()
+    torch.cuda.synchronize()
+    ms = a.elapsed_time(b) / reps
+    del src, dst
+    torch.cuda.empty_cache()
+    return round(2 * (1 << 30) / (ms * 1e-3) / 1e9, 1)
+
+
+def inference_leg(dev, frames, warmup):
+    """The headline metric's second figure: forward-only frames per second of the 3 M-Gaussian scene at
+    1920x1080 along its 300-camera orbit (every 7th camera), rays ended at T < 1e-4, tree built once and
+    reused (scripts/test.py:60-126).  A frame is view-dependent colour + primitive records + march."""
+    from raygaussx_amd.render_optix import compute_rgb
+    name = "c3_3M_1920x1080_fwd"
+    config, n, width, height = WORKLOADS[name]
+    cfg = scenes.CONFIGS[config]
+    d = {k: v.to(dev) for k, v in scenes.make_scene(config, n=n).items()}
+    cams = [scenes.make_camera(config, (7 * i) % cfg["n_cameras"], width=width, height=height).to(dev) for i in range(frames + warmup)]
+    structs = [u_ox.camera_struct(c) for c in cams]       # host copies of the camera constants: no sync per frame
+    t0 = time.perf_counter()
+    tree = u_ox.AccelerationStructure(n, dev).build_from_gaussians(d["positions"], d["scales"], d["quaternions"], d["densities"])
+    torch.cuda.synchronize()
+    stats = u_ox.new_stats(dev)
+
+    def frame(i, census=False):
+        rgb = compute_rgb(structs[i].eye, d["positions"], d["color_features"], None, None, None, 0, 3)
+        return u_ox.launch_pipeline_test(None, None, tree, None, None, cfg["dt_step"], cfg["dynamic_sampling"], cams[i],
+                                         d["densities"], rgb, d["positions"], d["scales"], d["quaternions"],
+                                         cfg["max_prim_slice"], t_eps=cfg["t_eps"], stats=stats if census else None)
+    for i in range(warmup):
+        frame(i)
+    torch.cuda.synchronize()
+    L.timing_enable(True)
+    t0 = time.perf_counter()
+    for i in range(frames):
+        frame(warmup + i)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    timing = L.timing_read()
+    L.timing_enable(False)
+    for i in range(frames):
+        frame(warmup + i, census=True)
+    torch.cuda.synchronize()
+    st = u_ox.read_stats(stats)
+    hits = st["hit_pairs"] / frames
+    n_rays = width * height
+    ms_kernel = timing["march_forward"][0] / max(timing["march_forward"][1], 1)
+    nbytes = 64.0 * hits + 12.0 * n_rays
+    gbps = nbytes / (ms_kernel * 1e-3) / 1e9
+    frame_bytes = nbytes + 300.0 * n
+    ms_frame = elapsed / frames * 1e3
+    traffic, source = stored_traffic(name, "march_forward")
+    return dict(value=round(frames / elapsed, 3), unit="frames/s", frames=frames, warmup=warmup, ms_per_frame=round(ms_frame, 4),
+                workload=name, gaussians=n, width=width, height=height, t_eps=cfg["t_eps"], dynamic_sampling=cfg["dynamic_sampling"],
+                frame="sh + pack + march fwd, 1 view, tree built once and reused",
+                roofline=dict(bound="hbm", kernel="k_march_fwd", achieved=round(gbps, 2), peak=HBM_PEAK_GBPS, unit="GB/s",
+                              frac=round(gbps / HBM_PEAK_GBPS, 5), traffic=traffic, traffic_source=source,
+                              kernel_ms=round(ms_kernel, 4), algorithmic_bytes=int(nbytes), hit_pairs_per_launch=int(hits)),
+                frame_roofline=dict(bytes_per_frame=int(frame_bytes), frac=round(frame_bytes / (ms_frame * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
+                                    roofline_fps=round(HBM_PEAK_GBPS * 1e9 / frame_bytes, 2)),
+                kernels_ms={k: round(v[0] / max(v[1], 1), 4) for k, v in timing.items() if v[1]})
 
 
 def _timed(fn, reps):
@@ -139,7 +238,10 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c4_1M_800x800", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-rays", type=int, default=16384, help="ray sample of the CPU baseline (0 = skip)")
+    ap.add_argument("--cpu-rays", type=int, default=262144, help="ray sample of the CPU baseline (0 = skip)")
+    ap.add_argument("--fps-frames", type=int, default=20,
+                    help="after the headline pass, frames of the 3 M-Gaussian 1920x1080 forward-only orbit to time for "
+                         "`fwd_fps_c3` (0 = skip; skipped for workloads other than the default)")
     ap.add_argument("--forward-only", action="store_true")
     ap.add_argument("--no-records", action="store_true",
                     help="backward searches the tree again instead of replaying the forward's hit-list record")
@@ -182,6 +284,7 @@ def main():
     params = [dscene[k].clone().requires_grad_(not args.forward_only) for k in names]
     n_cams = min(cfg["n_cameras"], 100)
     cams = [scenes.make_camera(config, i, width=width, height=height).to(dev) for i in range(n_cams)]
+    cam_structs = [u_ox.camera_struct(c) for c in cams]   # also caches each camera's host constants: no sync per step
     n_rays = width * height
     target = torch.rand(n_rays, 3, device=dev, generator=torch.Generator(dev).manual_seed(1))
     stats = u_ox.new_stats(dev)
@@ -206,7 +309,7 @@ def main():
             return out
         if inference:   # per frame: view-dependent colour, primitive records, march
             cam = cams[(7 * i) % n_cams]
-            rgb = compute_rgb(cam.camera_center, dscene["positions"], dscene["color_features"], None, None, None, 0, 3)
+            rgb = compute_rgb(cam_structs[(7 * i) % n_cams].eye, dscene["positions"], dscene["color_features"], None, None, None, 0, 3)
             return u_ox.launch_pipeline_test(None, None, tree, None, None, cfg["dt_step"], cfg["dynamic_sampling"], cam,
                                              dscene["densities"], rgb, dscene["positions"], dscene["scales"],
                                              dscene["quaternions"], cfg["max_prim_slice"], t_eps=cfg["t_eps"],
@@ -277,9 +380,10 @@ def main():
                                frac=round(gbps / HBM_PEAK_GBPS, 5))
     kname = max(per_kernel, key=lambda k: per_kernel[k]["kernel_ms"])
     dom = per_kernel[kname]
-    default_record = not (args.no_records or args.forward_only or args.rec_tile_words is not None)
+    default_record = not (args.no_records or args.rec_tile_words is not None)
+    traffic, traffic_source = stored_traffic(args.workload, kname) if default_record else (None, None)
     roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=dom["achieved"], peak=HBM_PEAK_GBPS, unit="GB/s", frac=dom["frac"],
-                    traffic=MEASURED_TRAFFIC_BYTES.get((args.workload, kname)) if default_record else None,
+                    traffic=traffic, traffic_source=traffic_source,
                     kernel_ms=dom["kernel_ms"], algorithmic_bytes=dom["algorithmic_bytes"],
                     hit_pairs_per_launch=int(hits_per_launch), march_kernels=per_kernel)
     # whole-step roofline-derived rate: all algorithmic bytes of one step at peak bandwidth
@@ -308,10 +412,23 @@ def main():
         out["atomics"] = dict(per_backward_launch=int(adds), unit="G atomic adds/s",
                               value=round(adds / (per_kernel["march_backward"]["kernel_ms"] * 1e-3) / 1e9, 3))
     out["views_in_flight"] = in_flight
+    rec_use = None if (inference or args.forward_only) else u_ox.record_use(cam_structs[0], dev)
+    out["memory"] = dict(peak_allocated_GB=round(torch.cuda.max_memory_allocated(dev) / 1e9, 3),
+                         record_allocated_GB=None if rec_use is None else round(rec_use[0] / 1e9, 3),
+                         record_used_GB=None if rec_use is None else round(rec_use[1] / 1e9, 3))
+    del params, dscene, target
+    gas = None
+    torch.cuda.empty_cache()
+    bw = copy_bandwidth(dev)
+    out["hbm_measured"] = dict(copy_GBps=bw, what="1 GiB device-to-device copy, bytes read + written",
+                               roofline_frac_of_measured=round(dom["achieved"] / bw, 5),
+                               step_frac_of_measured=round(out["step_roofline"]["achieved"] / bw, 5))
+    if args.fps_frames > 0 and args.workload == "c4_1M_800x800" and not args.forward_only:
+        out["fwd_fps_c3"] = inference_leg(dev, args.fps_frames, 3)
     if args.cpu_rays > 0:
         threads = min(16, os.cpu_count() or 1)
         out["cpu_baseline"] = cpu_baseline(scene, scenes.make_camera(config, 0, width=width, height=height), cfg,
-                                           args.cpu_rays if n <= 1_000_000 else min(args.cpu_rays, 4096), threads,
+                                           args.cpu_rays if n <= 1_000_000 else min(args.cpu_rays, 16384), threads,
                                            backward=not args.forward_only)
     else:
         out["cpu_baseline"] = None

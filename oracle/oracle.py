@@ -86,6 +86,18 @@ def set_step_scale(scale):
     lib().orc_set_step_scale(C.c_float(scale))
 
 
+def cull_build(prims):
+    """Build the oracle's optional bounding-volume tree over this primitive block (the timed CPU baseline
+    uses it; results are those of the brute force).  Keep ``prims`` alive and pass the same array to the
+    march calls; ``cull_free()`` drops the tree."""
+    assert prims.dtype == np.float32 and prims.flags["C_CONTIGUOUS"]
+    lib().orc_cull_build(C.c_int64(prims.shape[0]), _p(prims))
+
+
+def cull_free():
+    lib().orc_cull_free()
+
+
 def camera_struct(cam, supersampling=(1, 1)):
     """``cam`` exposes the reference Camera attributes read at optix_utils.py:258-266."""
     c = OrcCamera()

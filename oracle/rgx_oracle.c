@@ -378,19 +378,157 @@ static inline int segment_hit(float r1, float r2, float tmin, float tmax, float 
 
 typedef struct { Cand *c; int64_t n, cap; } CandList;
 
+static inline void cands_push(CandList *L, int32_t id, float r1, float r2)
+{
+    if (L->n == L->cap) {
+        L->cap = L->cap ? 2 * L->cap : 1024;
+        L->c = (Cand *)realloc(L->c, (size_t)L->cap * sizeof(Cand));
+    }
+    L->c[L->n].id = id; L->c[L->n].r1 = r1; L->c[L->n].r2 = r2;
+    L->n++;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Optional culling for the timed CPU baseline.  The brute-force loop below    */
+/* is the oracle proper: it evaluates the reference's predicate on every       */
+/* primitive.  With orc_cull_build() a bounding-volume tree over the           */
+/* primitives' k-sigma boxes (eye-relative, as the packed records are) feeds   */
+/* the same predicate only the primitives whose padded box the ray's line      */
+/* meets, and the survivors are put back into ascending index order, so the    */
+/* candidate lists -- and with them every result -- are those of the brute     */
+/* force (tests/test_oracle_geometry.py holds the two to each other).  The     */
+/* boxes are padded by 1e-5 of their distance from the eye, a hundred times    */
+/* what rounding lets the fp32 predicate accept outside the exact ellipsoid.   */
+typedef struct { float lo[3], hi[3]; int32_t a, b; } CullNode; /* inner: children a, b; leaf: a = first, b = -count */
+static struct { CullNode *nodes; int32_t *perm; int32_t n_nodes; const float *prims; int64_t N; } g_cull;
+
+static int cull_cmp(const void *x, const void *y)
+{
+    const uint64_t a = *(const uint64_t *)x, b = *(const uint64_t *)y;
+    return a < b ? -1 : a > b;
+}
+
+static int32_t cull_make(int32_t lo, int32_t hi, const float *boxes)
+{
+    const int32_t me = g_cull.n_nodes++;
+    CullNode *nd = &g_cull.nodes[me];
+    if (hi - lo <= 4) {
+        nd->a = lo; nd->b = -(hi - lo);
+        for (int c = 0; c < 3; ++c) { nd->lo[c] = INFINITY; nd->hi[c] = -INFINITY; }
+        for (int32_t j = lo; j < hi; ++j) {
+            const float *bx = boxes + 6 * (int64_t)g_cull.perm[j];
+            for (int c = 0; c < 3; ++c) { nd->lo[c] = fminf(nd->lo[c], bx[c]); nd->hi[c] = fmaxf(nd->hi[c], bx[3 + c]); }
+        }
+        return me;
+    }
+    const int32_t mid = lo + (hi - lo) / 2;
+    const int32_t a = cull_make(lo, mid, boxes), b = cull_make(mid, hi, boxes);
+    nd = &g_cull.nodes[me];
+    nd->a = a; nd->b = b;
+    for (int c = 0; c < 3; ++c) {
+        nd->lo[c] = fminf(g_cull.nodes[a].lo[c], g_cull.nodes[b].lo[c]);
+        nd->hi[c] = fmaxf(g_cull.nodes[a].hi[c], g_cull.nodes[b].hi[c]);
+    }
+    return me;
+}
+
+void orc_cull_free(void)
+{
+    free(g_cull.nodes); free(g_cull.perm);
+    memset(&g_cull, 0, sizeof g_cull);
+}
+
+/* Builds the tree for this primitive block; candidate searches on exactly this block (same   */
+/* pointer, same N) use it until orc_cull_free().                                             */
+void orc_cull_build(int64_t N, const float *prims)
+{
+    orc_cull_free();
+    if (N <= 0) return;
+    float *boxes = (float *)malloc(sizeof(float) * 6 * (size_t)N);
+    uint64_t *keys = (uint64_t *)malloc(sizeof(uint64_t) * (size_t)N);
+    float mn[3] = {INFINITY, INFINITY, INFINITY}, mx[3] = {-INFINITY, -INFINITY, -INFINITY};
+    int64_t live = 0;
+    for (int64_t i = 0; i < N; ++i) {
+        const float *p = prims + 16 * i;
+        if (!(p[7] == p[7])) continue; /* k is NaN below the density threshold: can never be hit */
+        f3 U, V, W;
+        quat_to_cols(p + 8, &U, &V, &W);
+        const float ax = 1.0f / p[4], ay = 1.0f / p[5], az = 1.0f / p[6]; /* k * scale */
+        const float h[3] = {sqrtf(U.x * U.x * ax * ax + V.x * V.x * ay * ay + W.x * W.x * az * az),
+                            sqrtf(U.y * U.y * ax * ax + V.y * V.y * ay * ay + W.y * W.y * az * az),
+                            sqrtf(U.z * U.z * ax * ax + V.z * V.z * ay * ay + W.z * W.z * az * az)};
+        const float c[3] = {-p[0], -p[1], -p[2]}; /* centre - eye */
+        const float pad = 1e-5f * (sqrtf(c[0] * c[0] + c[1] * c[1] + c[2] * c[2]) + fmaxf(h[0], fmaxf(h[1], h[2])) + 1.0f);
+        float *bx = boxes + 6 * i;
+        for (int a = 0; a < 3; ++a) {
+            bx[a] = c[a] - h[a] * 1.001f - pad; bx[3 + a] = c[a] + h[a] * 1.001f + pad;
+            mn[a] = fminf(mn[a], c[a]); mx[a] = fmaxf(mx[a], c[a]);
+        }
+        keys[live++] = (uint64_t)i; /* the code goes into the upper bits below */
+    }
+    for (int64_t j = 0; j < live; ++j) {
+        const int64_t i = (int64_t)keys[j];
+        const float *p = prims + 16 * i;
+        uint64_t code = 0;
+        const float c[3] = {-p[0], -p[1], -p[2]};
+        uint32_t q[3];
+        for (int a = 0; a < 3; ++a) {
+            const float u = (c[a] - mn[a]) / fmaxf(mx[a] - mn[a], 1e-30f);
+            q[a] = (uint32_t)fminf(fmaxf(u * 1023.0f, 0.0f), 1023.0f);
+        }
+        for (int b = 0; b < 10; ++b)
+            for (int a = 0; a < 3; ++a) code |= (uint64_t)((q[a] >> b) & 1u) << (3 * b + a);
+        keys[j] = code << 32 | (uint64_t)i;
+    }
+    qsort(keys, (size_t)live, sizeof(uint64_t), cull_cmp);
+    g_cull.perm = (int32_t *)malloc(sizeof(int32_t) * (size_t)(live > 0 ? live : 1));
+    for (int64_t j = 0; j < live; ++j) g_cull.perm[j] = (int32_t)(keys[j] & 0xffffffffu);
+    g_cull.nodes = (CullNode *)malloc(sizeof(CullNode) * (size_t)(live > 0 ? live : 1));
+    g_cull.n_nodes = 0;
+    if (live > 0) cull_make(0, (int32_t)live, boxes);
+    g_cull.prims = prims; g_cull.N = N;
+    free(boxes); free(keys);
+}
+
+static int cand_cmp(const void *x, const void *y) { return ((const Cand *)x)->id - ((const Cand *)y)->id; }
+
+static void cands_build_culled(CandList *L, const float *prims, f3 dir)
+{
+    int32_t stack[128];
+    int sp = 0;
+    if (g_cull.n_nodes > 0) stack[sp++] = 0;
+    const float d[3] = {dir.x, dir.y, dir.z};
+    while (sp > 0) {
+        const CullNode *nd = &g_cull.nodes[stack[--sp]];
+        float tn = -INFINITY, tf = INFINITY; /* the whole line: the predicate's roots do not depend on the interval */
+        int miss = 0;
+        for (int a = 0; a < 3 && !miss; ++a) {
+            if (d[a] == 0.0f) { miss = nd->lo[a] > 0.0f || nd->hi[a] < 0.0f; continue; }
+            const float inv = 1.0f / d[a];
+            const float t0 = nd->lo[a] * inv, t1 = nd->hi[a] * inv;
+            tn = fmaxf(tn, fminf(t0, t1)); tf = fminf(tf, fmaxf(t0, t1));
+        }
+        if (miss || tn > tf) continue;
+        if (nd->b < 0) {
+            for (int32_t j = nd->a; j < nd->a - nd->b; ++j) {
+                const int32_t i = g_cull.perm[j];
+                float r1, r2;
+                if (line_roots(prims + 16 * (int64_t)i, dir, &r1, &r2)) cands_push(L, i, r1, r2);
+            }
+        } else if (sp + 2 <= 128) { /* depth <= log2(N) + 1 */
+            stack[sp++] = nd->a; stack[sp++] = nd->b;
+        }
+    }
+    qsort(L->c, (size_t)L->n, sizeof(Cand), cand_cmp); /* ascending index, as the brute force lists them */
+}
+
 static void cands_build(CandList *L, int64_t N, const float *prims, f3 dir)
 {
     L->n = 0;
+    if (g_cull.nodes && g_cull.prims == prims && g_cull.N == N) { cands_build_culled(L, prims, dir); return; }
     for (int64_t i = 0; i < N; ++i) {
         float r1, r2;
-        if (line_roots(prims + 16 * i, dir, &r1, &r2)) {
-            if (L->n == L->cap) {
-                L->cap = L->cap ? 2 * L->cap : 1024;
-                L->c = (Cand *)realloc(L->c, (size_t)L->cap * sizeof(Cand));
-            }
-            L->c[L->n].id = (int32_t)i; L->c[L->n].r1 = r1; L->c[L->n].r2 = r2;
-            L->n++;
-        }
+        if (line_roots(prims + 16 * i, dir, &r1, &r2)) cands_push(L, (int32_t)i, r1, r2);
     }
 }
 

@@ -220,11 +220,51 @@ def fit_tile_words(cam, tile_words, budget_bytes):
     return lists + slots * REC_SLOT_WORDS if (tile_words > lists and slots >= 1) else lists
 
 
+# What the forward launches of one image size actually took from the sample-sum pool, so that the next
+# record of that size is allocated for the need instead of for 64 slots per tile:
+# (device, width, height) -> {"pinned": host int32[1], "event", "pending", "need": slots of the last views,
+#                             "slots": the pool size in use, "allocated": bytes of the last record}
+_rec_usage = {}
+REC_POOL_MARGIN = 1.05        # pool = this times the largest need of the last views ...
+REC_POOL_STEP = 1 << 15       # ... rounded up to a multiple of this many slots (1 GiB), so that the size stays put
+REC_POOL_HISTORY = 8
+
+
+def _pool_geometry(cam):
+    ntiles = ((cam.width + 7) // 8) * ((cam.height + 7) // 8)
+    return ntiles, ntiles * REC_LIST_WORDS * 4        # tiles, bytes of the hit-list regions (the pool header follows)
+
+
 def new_records(cam, device, tile_words=REC_TILE_WORDS, budget_bytes=None):
     """Buffer for the record of one forward launch (see rgx_march_records_bytes), or None when no
-    record fits the budget (default: REC_MEMORY_SHARE of the device's memory) or the allocator."""
+    record fits the budget or the allocator.  The budget defaults to REC_MEMORY_SHARE of the device's
+    memory and at most 80 % of what is free now.  With the default ``tile_words`` the pool of sample
+    sums is sized from what the last forward launches of this image size took from it
+    (``note_record_use``) instead of the 64 slots per tile of a first call: tiles that find the pool
+    empty are replayed from their hit lists alone, so a guess that is too small costs time, not
+    correctness, and the next record grows."""
     if budget_bytes is None:
-        budget_bytes = int(REC_MEMORY_SHARE * torch.cuda.get_device_properties(device).total_memory)
+        free, total = torch.cuda.mem_get_info(device)
+        budget_bytes = int(min(REC_MEMORY_SHARE * total, 0.8 * free))
+    use = _rec_usage.get((str(device), cam.width, cam.height))
+    if tile_words == REC_TILE_WORDS and use is not None and use["need"]:
+        _read_record_use(use)
+        ntiles, head = _pool_geometry(cam)
+        have = use.get("slots", 0)
+        need = max(use["need"])
+        # a launch that ran the pool dry stops counting tile by tile, so its count is a lower bound: grow faster
+        want = int(need * (1.5 if have and need >= have else REC_POOL_MARGIN)) + 1
+        if want > have or want * 1.5 < have:      # grow when short; shrink only when far too large
+            have = (want + REC_POOL_STEP - 1) // REC_POOL_STEP * REC_POOL_STEP
+        have = min(have, 64 * ntiles)
+        nbytes = head + 256 + have * REC_SLOT_WORDS * 4
+        if have > ntiles and nbytes <= budget_bytes:
+            try:
+                rec = torch.empty(nbytes, dtype=torch.uint8, device=device)
+                use["slots"] = have
+                return rec
+            except torch.cuda.OutOfMemoryError:
+                pass
     words = fit_tile_words(cam, tile_words, budget_bytes)
     while words:
         try:
@@ -232,6 +272,48 @@ def new_records(cam, device, tile_words=REC_TILE_WORDS, budget_bytes=None):
         except torch.cuda.OutOfMemoryError:
             words = REC_LIST_WORDS if words > REC_LIST_WORDS else 0   # try the hit lists alone, then give up
     return None
+
+
+def _read_record_use(use):
+    if use["pending"] and use["event"].query():
+        use["pending"] = False
+        use["need"] = (use["need"] + [int(use["pinned"][0])])[-REC_POOL_HISTORY:]
+
+
+def note_record_use(records, cam, device):
+    """After a forward launch that wrote ``records``: queue a 4-byte copy of the pool's bump counter
+    (the slots the launch asked for, also beyond the pool's end) to pinned host memory.  Nothing waits
+    for it; the next ``new_records`` of this image size reads it."""
+    ntiles, head = _pool_geometry(cam)
+    if records is None or records.numel() < head + 256 + REC_SLOT_WORDS * 4 or records.numel() // 4 // ntiles < REC_LIST_WORDS + REC_SLOT_WORDS:
+        return
+    key = (str(device), cam.width, cam.height)
+    use = _rec_usage.get(key)
+    if use is None:
+        if len(_rec_usage) >= 64:
+            del _rec_usage[next(iter(_rec_usage))]
+        use = _rec_usage[key] = dict(pinned=torch.zeros(1, dtype=torch.int32).pin_memory(), event=torch.cuda.Event(),
+                                     pending=False, need=[])
+    use["allocated"] = records.numel()
+    _read_record_use(use)
+    if use["pending"]:
+        return                                  # the previous copy has not landed yet: leave its buffer alone
+    use["pinned"].copy_(records[head:head + 4].view(torch.int32), non_blocking=True)
+    use["event"].record(torch.cuda.current_stream(device))
+    use["pending"] = True
+
+
+def record_use(cam, device):
+    """(bytes allocated for the last record of this image size, bytes of it the last launch read back used:
+    hit-list regions + sample-sum slots), or None before the first launch has reported."""
+    use = _rec_usage.get((str(device), cam.width, cam.height))
+    if use is None:
+        return None
+    _read_record_use(use)
+    if not use["need"]:
+        return None
+    ntiles, head = _pool_geometry(cam)
+    return use["allocated"], head + 256 + use["need"][-1] * REC_SLOT_WORDS * 4
 
 
 def march_forward(gas, cam, prims, dt_step, dynamic_sampling, max_prim_slice, white_background,

@@ -126,6 +126,7 @@ class RenderOptixFunction(torch.autograd.Function):
         ray_colors = u_ox.march_forward(gas, cam, prims, settings.dt_step, settings.dynamic_sampling,
                                         settings.max_prim_slice, settings.white_background, settings.t_eps,
                                         settings.stats, records)
+        u_ox.note_record_use(records, cam, dev)
         ctx.records = records
         ctx.settings = settings
         ctx.cam = cam

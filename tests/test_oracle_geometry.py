@@ -269,3 +269,34 @@ def test_knn3_mean_distance_matches_a_kd_tree(orc):
         np.testing.assert_allclose(orc.dist2_knn3(p), want, rtol=2e-6, atol=1e-12)
     two = orc.dist2_knn3(np.array([[0, 0, 0], [1, 0, 0]], np.float32))
     assert np.isinf(two).all()                 # (1 + FLT_MAX + FLT_MAX) / 3 overflows, as in the reference
+
+
+def test_culled_candidate_search_equals_the_brute_force(orc):
+    """The bounding-volume tree the timed CPU baseline uses (orc_cull_build) must change nothing: the
+    candidate lists are those of the loop over all primitives, so images, counters, hit lists and
+    gradients are equal in every bit -- for an object scene, for the heavy-tailed one with the camera
+    inside the cloud, with invisible Gaussians (k undefined) and with axis-parallel rays."""
+    from raygaussx_amd import scenes
+    for config, n, w, h, mult in ((0, 3000, 40, 32, 2.0), (2, 8000, 36, 28, 3.0), (1, 5000, 33, 33, 4.0)):
+        sc = scenes.scene_to_numpy(scenes.make_scene(config, n=n, sh_degree=1, seed=50 + config))
+        sc["scales"] = sc["scales"] * mult
+        sc["densities"][::7] = 0.05                                  # below the threshold: never hit
+        cam = scenes.look_at_camera((3.0, 0.0, 0.0), fov_x_deg=30, width=w, height=h) if config == 1 else \
+            scenes.make_camera(config, 2, width=w, height=h)
+        cfg = scenes.CONFIGS[config]
+        img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], cfg["dynamic_sampling"], 512)
+        dloss = np.random.default_rng(config).normal(size=img.shape).astype(np.float32)
+        g, _ = orc.march_backward(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], img, dloss)
+        slabs, _ = orc.march_trace(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], (h // 2) * w + w // 2)
+        orc.cull_build(ctx["prims"])
+        try:
+            img2, st2 = orc.march_forward(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"])
+            g2, _ = orc.march_backward(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], img, dloss)
+            slabs2, _ = orc.march_trace(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], (h // 2) * w + w // 2)
+        finally:
+            orc.cull_free()
+        assert st == st2 and st["hit_pairs"] > 2000
+        assert np.array_equal(img, img2)
+        for k in g:
+            assert np.array_equal(g[k], g2[k]), k
+        assert len(slabs) == len(slabs2) and all(a[:4] == b[:4] and np.array_equal(a[4], b[4]) for a, b in zip(slabs, slabs2))

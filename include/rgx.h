@@ -123,6 +123,13 @@ int rgx_build(const float *pos, const float *scale, const float *quat, const flo
  * create_acceleration_structure(ctx, bboxes) (optix_utils.py:139-142). */
 int rgx_build_aabbs(const float *bboxes, int64_t n, void *ws, size_t ws_bytes, void *stream);
 
+/* Replaces update_acceleration_structure(gas, bboxes) (optix_utils.py:144-146; OptiX's
+ * accel update): new boxes for the same Gaussians into a workspace that rgx_build / rgx_build_aabbs
+ * built for this n.  The tree keeps its shape (sorted order, children); leaf and internal boxes and
+ * the scene box are recomputed.  About a third of a build's time; queries stay exact however far the
+ * Gaussians moved, the tree only culls worse the further they did. */
+int rgx_refit_aabbs(const float *bboxes, int64_t n, void *ws, size_t ws_bytes, void *stream);
+
 /* Synchronous read-back of the scene bbox held in a built workspace
  * (host out[6] = min xyz, max xyz); what bb_min.get()/bb_max.get() returned at
  * optix_utils.py:254-255.  Waits for `stream`. */

@@ -548,6 +548,37 @@ static int build_impl(const float *pos, const float *scale, const float *quat, c
     return RGX_OK;
 }
 
+// Refit: the tree's shape (children, parents, sorted order) stays as the last build into `ws` left it;
+// leaf boxes are taken from `bboxes`, internal boxes and the scene box recomputed bottom-up.
+extern "C" int rgx_refit_aabbs(const float *bboxes, int64_t n, void *ws, size_t ws_bytes, void *stream)
+{
+    if (n < 0 || n > 0x3fffffff || !ws || (n > 0 && !bboxes)) return RGX_EINVAL;
+    const DeviceScope on_device(ws);
+    const WsLayout L = rgx_ws_layout(n);
+    if (ws_bytes < L.total || ((uintptr_t)ws & 255u)) return RGX_EWORKSPACE;
+    hipStream_t s = (hipStream_t)stream;
+    char *w = (char *)ws;
+    WsHeader *hdr = (WsHeader *)(w + L.header);
+    float *boxes = (float *)(w + L.aabb);
+    const uint32_t *order = (const uint32_t *)(w + L.vals0);
+    Node *nodes = (Node *)(w + L.nodes);
+    int32_t *parent = (int32_t *)(w + L.parent), *right = (int32_t *)(w + L.right), *flags = (int32_t *)(w + L.flags);
+    const int32_t *other_end = (const int32_t *)(w + L.keys1); // left there by the build
+    void *span = rgx_span_begin(RGX_T_BUILD, s);
+    hipLaunchKernelGGL(k_init_header, dim3(1), dim3(64), 0, s, hdr, n);
+    if (n > 0) {
+        hipLaunchKernelGGL(k_take_boxes, grid_for(n, 256), dim3(256), 0, s, bboxes, n, boxes, hdr->bb_min_enc, hdr->bb_max_enc);
+        hipLaunchKernelGGL(k_finish_bbox, dim3(1), dim3(64), 0, s, hdr, (float *)nullptr, (float *)nullptr);
+        hipLaunchKernelGGL(k_leaves, grid_for(n, 256), dim3(256), 0, s, boxes, order, n, nodes, parent, flags);
+        if (n > 1) hipLaunchKernelGGL(k_refit, grid_for(n, 256), dim3(256), 0, s, n, nodes, parent, right, other_end, flags);
+        hipLaunchKernelGGL(k_skip_links, grid_for(2 * n - 1, 256), dim3(256), 0, s, n, nodes, parent, right);
+    }
+    hipLaunchKernelGGL(k_mark_built, dim3(1), dim3(1), 0, s, hdr);
+    rgx_span_end(span, s);
+    RGX_LAUNCH_CHECK();
+    return RGX_OK;
+}
+
 extern "C" int rgx_build_layout(int64_t n, size_t *host_out6)
 {
     if (n < 0 || n > 0x3fffffff || !host_out6) return RGX_EINVAL;

@@ -72,7 +72,11 @@ class AccelerationStructure:
         return self
 
     def update(self, bboxes):
-        return self.build_from_boxes(L.f32(bboxes))
+        """New boxes for the same Gaussians: refit (the tree keeps its shape), as OptiX's accel update does."""
+        bboxes = L.f32(bboxes)
+        L.check(L.lib().rgx_refit_aabbs(L.ptr(bboxes), C.c_int64(self.n), L.ptr(self.ws), C.c_size_t(self.ws.numel()),
+                                        L.stream(self.device)))
+        return self
 
     def scene_bbox(self):
         out = (C.c_float * 6)()
@@ -120,7 +124,7 @@ def create_acceleration_structure(ctx, bboxes):
 
 
 def update_acceleration_structure(gas, bboxes):
-    """optix_utils.py:144-146 (rebuilds in place; the build is cheap enough not to need a refit path)."""
+    """optix_utils.py:144-146: refit of an existing acceleration structure to new boxes."""
     gas.update(bboxes)
 
 

@@ -1156,6 +1156,7 @@ struct ReplayLds {
     float *acc;        // [RGX_NSUM][RGX_CCAP], component-major so that different slots fall in different banks
     uint32_t *pid;     // [RGX_CCAP]: the window's Gaussians by slot; top bit: the slot has something in acc
     float *frame;      // [9][RGX_CCAP]: rotation columns U, V, W of the window's Gaussians
+    uint8_t *rowlist;  // [4][RGX_CCAP]: the slot lists of the LISTS item whose gradient pass is running
 };
 
 __device__ __forceinline__ void replay_flush(const MarchParams &P, const ReplayLds &RL)
@@ -1216,6 +1217,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
     const int len = row == 0 ? l0 : row == 1 ? l1 : row == 2 ? l2 : l3;
     const uint8_t *slots = (const uint8_t *)(it + 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0));
     const uint32_t *masks = it + 8 + q0 + q1 + q2 + q3 + lane; // word w of this lane: masks[w * 64]
+    (void)RL.rowlist;
     if constexpr (WALK == WALK_NONE) {
         const int nwr = run ? min((len + 31) >> 5, nw) : 0;
         if (COUNT)
@@ -1242,6 +1244,14 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
         }
     } else {
         const int maxlen = min(max(max(l0, l1), max(l2, l3)), nw * 32);
+        // the rows' slot lists go to LDS first: every trip starts by looking its slot up, and from memory that
+        // look-up is a round trip at the head of the trip's chain of dependent loads
+        {
+            uint32_t *dst = (uint32_t *)(RL.rowlist + row * RGX_CCAP);
+            for (int i = lane & 15; i < min((len + 3) >> 2, RGX_CCAP / 4); i += 16) dst[i] = ((const uint32_t *)slots)[i];
+            __syncthreads();
+            slots = RL.rowlist + row * RGX_CCAP;
+        }
         uint32_t bits = 0;
         for (int i = 0; i < maxlen; ++i) {
             if ((i & 31) == 0) bits = masks[(i >> 5) * 64];
@@ -1249,7 +1259,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
             const bool hit = run && live && ((bits >> (i & 31)) & 1u);
             if (COUNT && hit) ++p0;
             if (__ballot(hit)) {
-                const int slot = live ? min((int)slots[i], RGX_CCAP - 1) : 0;
+                const int slot = live ? min((int)slots[min(i, RGX_CCAP - 1)], RGX_CCAP - 1) : 0;
                 const int32_t pid = (int32_t)(RL.pid[slot] & ~RGX_SLOT_TOUCHED);
                 body(Entry<false>{(const float4 *)(RL.frame + slot), P.prims + pid, pid, slot}, hit, live, Half<0>{});
             }
@@ -1730,7 +1740,8 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
     __shared__ float s_acc[REPLAY ? RGX_NSUM * RGX_CCAP : 1];
     __shared__ uint32_t s_pid[REPLAY ? RGX_CCAP : 1];
     __shared__ float s_frame[REPLAY ? 9 * RGX_CCAP : 1];
-    const ReplayLds RL = {s_acc, s_pid, s_frame};
+    __shared__ __align__(4) uint8_t s_rowlist[REPLAY ? 4 * RGX_CCAP : 4];
+    const ReplayLds RL = {s_acc, s_pid, s_frame, s_rowlist};
     if constexpr (REPLAY) {
         for (int i = lane; i < RGX_NSUM * RGX_CCAP; i += 64) s_acc[i] = 0.f;
         for (int i = lane; i < RGX_CCAP; i += 64) s_pid[i] = 0u;

@@ -22,6 +22,7 @@
 // The first-hit query (once per ray, and after an empty slab) runs on the same candidate tables.
 // The per-lane skip-link queries below serve the segment test hooks (arbitrary rays).
 #include "rgx_device.h"
+#include <hip/hip_fp16.h>
 
 #include <mutex>
 #include <type_traits>
@@ -1694,13 +1695,21 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
     flush_stats(P.stats, cn);
 }
 
-// sum over the 16 lanes of each row, left in every lane of the row
+// sum over the 16 lanes of each row, left in every lane of the row.  (Every lane of these four
+// patterns reads a lane of its own row, so bound_ctrl changes nothing but the instruction: without
+// it the last stage, whose add the compiler sinks into the one-lane-per-row branch that uses it,
+// costs a zeroed register and a move per value.)
+template <int CTRL>
+__device__ __forceinline__ float row_take(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float row_sum(float v)
 {
-    v += dpp_f<0xB1, 0xf>(0.f, v);  // quad_perm [1,0,3,2]
-    v += dpp_f<0x4E, 0xf>(0.f, v);  // quad_perm [2,3,0,1]
-    v += dpp_f<0x141, 0xf>(0.f, v); // row_half_mirror
-    v += dpp_f<0x140, 0xf>(0.f, v); // row_mirror
+    v += row_take<0xB1>(v);  // quad_perm [1,0,3,2]
+    v += row_take<0x4E>(v);  // quad_perm [2,3,0,1]
+    v += row_take<0x141>(v); // row_half_mirror
+    v += row_take<0x140>(v); // row_mirror
     return v;
 }
 
@@ -1805,10 +1814,17 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                 const float *col = (const float *)slot + RGX_BUFFER_SIZE * 64 + lane * 3;
 #pragma unroll
                 for (int i = 0; i < RGX_BUFFER_SIZE; ++i) PA[i] = __builtin_nontemporal_load(dens + i * 64);
+#ifdef RGX_PROBE_FP16_SUMS
+                // probe: what half-precision storage of the colour sums would cost in accuracy (values rounded to
+                // binary16 and back; the density sums stay exact, the transmittance must replay bit for bit)
+                auto h16 = [](float v) { return __half2float(__float2half(v)); };
+#else
+                auto h16 = [](float v) { return v; };
+#endif
 #pragma unroll
                 for (int i = 0; i < RGX_BUFFER_SIZE; ++i)
-                    PB[i] = fmaf(g.x, __builtin_nontemporal_load(col + i * 192),
-                                 fmaf(g.y, __builtin_nontemporal_load(col + i * 192 + 1), g.z * __builtin_nontemporal_load(col + i * 192 + 2)));
+                    PB[i] = fmaf(g.x, h16(__builtin_nontemporal_load(col + i * 192)),
+                                 fmaf(g.y, h16(__builtin_nontemporal_load(col + i * 192 + 1)), g.z * h16(__builtin_nontemporal_load(col + i * 192 + 2))));
             };
             // (2) prefix: PA <- a_k, PB <- (T_k e_k - D_k) dt - a_k e_k   (so X_k = PB + PA * g.c_i);
             // it always covers all 32 samples (330-352)

@@ -57,6 +57,7 @@ def test_ray_sample_against_the_oracle(gx, orc, big):
     assert out["stats_fwd"]["overflow_rays"] == 0
     for k in PARAMS:
         cos, rel = gx.cos_rel(out["grads"][k], og[k])
+        print(f"{k}: 1 - cos {1 - cos:.2e}, rel {rel:.2e}", flush=True)
         assert cos >= COS_MIN and rel <= REL_MAX, (k, cos, rel)
 
 

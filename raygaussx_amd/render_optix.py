@@ -113,7 +113,12 @@ class RenderOptixFunction(torch.autograd.Function):
         stale = gas is None or not isinstance(gas, u_ox.AccelerationStructure) or gas.n != n or gas.device != dev
         if stale:
             gas = u_ox.AccelerationStructure(n, dev)
-        if stale or not settings.gas_is_current:
+        if settings.update and not stale:
+            # render_optix.py:114-115: the existing structure takes the new boxes and keeps its shape
+            if not settings.gas_is_current:
+                boxes, _, _ = u_ox.ellipsoids_bbox_from_quat(normalized_quaternions, positions, scales, densities)
+                u_ox.update_acceleration_structure(gas, boxes)
+        elif stale or not settings.gas_is_current:
             gas.build_from_gaussians(positions, scales, normalized_quaternions, densities)
         settings.gas = gas
         order_sh = int(round(math.sqrt(color_features.shape[2]))) - 1   # render_optix.py:119

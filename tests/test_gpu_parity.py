@@ -1056,3 +1056,43 @@ def test_update_acceleration_structure_refits_the_tree(gx, orc):
     for k in ("hit_pairs", "slabs", "empty_slabs", "rays_hit"):
         assert got[k] == st[k], k
     assert st["hit_pairs"] > 20000 and np.abs(img.cpu().numpy() - want).max() <= IMG_TOL
+
+
+@pytest.mark.gpu
+def test_settings_update_refits_inside_the_render_function(gx):
+    """render_optix.py:114-117: with ``settings.update`` the forward hands the new boxes to the
+    existing acceleration structure instead of creating one.  A loop that moves the Gaussians between
+    two views renders the second view on the refitted tree; image and gradients equal those of a
+    forward that builds a new tree (same hit sets; the sums run in another order)."""
+    from raygaussx_amd.render_optix import RenderOptixFunction, default_settings
+    sc = scenes.scene_to_numpy(scenes.make_scene(0, n=5000, sh_degree=1, seed=21))
+    sc["scales"] = sc["scales"] * 2.0
+    cam = scenes.make_camera(0, 2, width=64, height=48).to(gx.DEV)
+    rng = np.random.default_rng(8)
+    moved = dict(sc)
+    moved["positions"] = (sc["positions"] + rng.normal(size=sc["positions"].shape).astype(np.float32) * 0.03).astype(np.float32)
+    dl = torch.from_numpy(rng.normal(size=(64 * 48, 3)).astype(np.float32)).to(gx.DEV)
+    names = ("positions", "scales", "quaternions", "densities", "color_features")
+    n = sc["positions"].shape[0]
+    empty = (torch.zeros(n, 3, 0, device=gx.DEV), torch.zeros(n, 0, device=gx.DEV), torch.zeros(n, 0, 3, device=gx.DEV))
+
+    def view(scene, settings):
+        d = gx.to_dev(scene)
+        args = [d[k].clone().requires_grad_(True) for k in names]
+        img = RenderOptixFunction.apply(*args, *empty, settings)
+        img.backward(dl)
+        return img.detach().cpu().numpy(), [a.grad.cpu().numpy() for a in args]
+
+    _step("first view builds, second refits")
+    s_upd = default_settings(cam, 0.0025, False, 2048)
+    view(sc, s_upd)
+    tree, order = s_upd.gas, s_upd.gas.order().cpu().numpy()
+    s_upd.update = True
+    img_u, g_u = view(moved, s_upd)
+    assert s_upd.gas is tree and np.array_equal(tree.order().cpu().numpy(), order)       # refitted, not rebuilt
+    s_new = default_settings(cam, 0.0025, False, 2048)
+    img_n, g_n = view(moved, s_new)
+    assert np.abs(img_n).max() > 0.1 and np.abs(img_u - img_n).max() <= 1e-5
+    for k, a, b in zip(names, g_u, g_n):
+        c, r = gx.cos_rel(a, b)
+        assert c >= 0.99999 and r <= 1e-4, (k, c, r)

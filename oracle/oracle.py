@@ -297,9 +297,12 @@ def morton_order(pos):
 # --------------------------------------------------------------------------- #
 # Whole-operator restatement (render_optix.py:94-199)
 def render_forward(scene, cam, dt_step, dynamic_sampling, max_prim_slice, white_background=True,
-                   supersampling=(1, 1), t_eps=TRANSMITTANCE_EPSILON, ray_ids=None):
+                   supersampling=(1, 1), t_eps=TRANSMITTANCE_EPSILON, ray_ids=None, cull=False):
     """scene: dict of numpy arrays positions, scales, quaternions, densities,
-    color_features (N,3,K) [+ sph_gauss_features, bandwidth_sharpness, lobe_axis]."""
+    color_features (N,3,K) [+ sph_gauss_features, bandwidth_sharpness, lobe_axis].
+    ``cull``: find candidates through the bounding-volume tree (same results, faster on large
+    scenes); the tree belongs to this view's primitive block and stays until ``render_backward``
+    with the returned context, or ``cull_free()``."""
     cs = camera_struct(cam, supersampling)
     ms = march_struct(dt_step, dynamic_sampling, max_prim_slice, white_background, t_eps)
     eye = np.asarray(cam.camera_center, np.float32)
@@ -308,14 +311,18 @@ def render_forward(scene, cam, dt_step, dynamic_sampling, max_prim_slice, white_
                      scene.get("bandwidth_sharpness"), scene.get("lobe_axis"))
     prims = pack_prims(eye, scene["positions"], scene["scales"], scene["quaternions"],
                        scene["densities"], rgb)
+    if cull:
+        cull_build(prims)
     img, stats = march_forward(cs, ms, bmin, bmax, prims, ray_ids)
-    ctx = dict(cs=cs, ms=ms, bmin=bmin, bmax=bmax, rgb=rgb, prims=prims, eye=eye, ray_ids=ray_ids)
+    ctx = dict(cs=cs, ms=ms, bmin=bmin, bmax=bmax, rgb=rgb, prims=prims, eye=eye, ray_ids=ray_ids, cull=cull)
     return img, stats, ctx
 
 
 def render_backward(scene, ctx, ray_colors, dloss):
     g, stats = march_backward(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"],
                               ray_colors, dloss, ctx["ray_ids"])
+    if ctx.get("cull"):
+        cull_free()
     dsh, dpos_dir, dsg, dsharp, daxis = sh_backward(
         ctx["eye"], scene["positions"], scene["color_features"], g["drgb"],
         scene.get("sph_gauss_features"), scene.get("bandwidth_sharpness"), scene.get("lobe_axis"))

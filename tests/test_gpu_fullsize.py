@@ -371,3 +371,63 @@ def test_heavy_tailed_scene_at_3M_gaussians(gx, orc):
     img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], True, cfg["max_prim_slice"], ray_ids=ids)
     _step("configs[2]: 3 M Gaussians, 1237x822, adaptive step, forward + backward")
     _adaptive_gates(gx, orc, sc, cam, cfg, ids, img, st, ctx, dloss)
+
+
+@pytest.mark.timeout(300)
+def test_accumulation_window_perturb_and_rebuild_at_1M(gx, orc):
+    """The loop of the 1 M-Gaussian configuration as a training script runs it: the gradients of the
+    20 views of a window accumulate in .grad (the tree built for the first view and marked current for
+    the others, no statistics block: the kernels a training loop launches), the Gaussians are then
+    perturbed, and the next window rebuilds the tree in place.  The accumulated gradients of both
+    windows face the sum of the oracle's per-view gradients, dL/dimage being non-zero on a ray
+    sample per view."""
+    from raygaussx_amd.render_optix import RenderOptixFunction, default_settings
+    cfg = scenes.CONFIGS[4]
+    sc = scenes.scene_to_numpy(scenes.make_scene(4, n=N))
+    sc = {k: sc[k] for k in PARAMS}
+    rng = np.random.default_rng(31)
+    empty = (torch.zeros(N, 3, 0, device=gx.DEV), torch.zeros(N, 0, device=gx.DEV), torch.zeros(N, 0, 3, device=gx.DEV))
+
+    def window(scene, cams, gas, n_rays):
+        params = [torch.from_numpy(scene[k]).to(gx.DEV).requires_grad_(True) for k in PARAMS]
+        want = {k: np.zeros(scene[k].shape, np.float64) for k in PARAMS}
+        worst = 0.0
+        for i, ci in enumerate(cams):
+            cam = scenes.make_camera(4, ci, width=W, height=H)
+            ids = np.sort(rng.choice(W * H, n_rays, replace=False)).astype(np.int64)
+            dloss = np.zeros((W * H, 3), np.float32)
+            dloss[ids] = rng.normal(size=(n_rays, 3)).astype(np.float32)
+            s = default_settings(cam.to(gx.DEV), cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"], gas=gas)
+            s.gas_is_current = i > 0
+            img = RenderOptixFunction.apply(*params, *empty, s)
+            img.backward(torch.from_numpy(dloss).to(gx.DEV))
+            gas = s.gas
+            o_img, _, ctx = orc.render_forward(scene, cam, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
+                                               ray_ids=ids, cull=True)
+            og, _ = orc.render_backward(scene, ctx, o_img, dloss)
+            worst = max(worst, float(np.abs(img.detach().cpu().numpy()[ids] - o_img[ids]).max()))
+            for k in PARAMS:
+                want[k] += og[k]
+        torch.cuda.synchronize()
+        return {k: p.grad.cpu().numpy() for k, p in zip(PARAMS, params)}, want, worst, gas
+
+    _step("window of 20 views, one tree")
+    got, want, worst, gas = window(sc, list(range(20)), None, 24)
+    assert worst <= IMG_TOL
+    for k in PARAMS:
+        cos, rel = gx.cos_rel(got[k], want[k])
+        print(f"window 1 {k}: 1 - cos {1 - cos:.2e}, rel {rel:.2e}", flush=True)
+        assert cos >= COS_MIN and rel <= REL_MAX, (k, cos, rel)
+    # an optimiser step's worth of change, then the next window: same workspace, tree rebuilt in place
+    moved = dict(sc)
+    moved["positions"] = (sc["positions"] + rng.normal(size=sc["positions"].shape).astype(np.float32) * 2e-3).astype(np.float32)
+    moved["scales"] = (sc["scales"] * np.exp(rng.normal(size=sc["scales"].shape) * 0.02)).astype(np.float32)
+    moved["densities"] = (sc["densities"] * np.exp(rng.normal(size=sc["densities"].shape) * 0.02)).astype(np.float32)
+    _step("window of 4 views after the perturbation, tree rebuilt in place")
+    ws_before = gas.ws.data_ptr()
+    got, want, worst, gas2 = window(moved, [20, 21, 22, 23], gas, 48)
+    assert gas2 is gas and gas.ws.data_ptr() == ws_before and worst <= IMG_TOL
+    for k in PARAMS:
+        cos, rel = gx.cos_rel(got[k], want[k])
+        print(f"window 2 {k}: 1 - cos {1 - cos:.2e}, rel {rel:.2e}", flush=True)
+        assert cos >= COS_MIN and rel <= REL_MAX, (k, cos, rel)

@@ -47,20 +47,43 @@ HBM_PEAK_GBPS = 8000.0
 PROFILES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles")
 
 
+def _stored(tag, workload, kernel_key):
+    import glob
+    import re
+    for path in sorted(glob.glob(os.path.join(PROFILES, "*.md"))):
+        for line in open(path):
+            m = re.match(r"\s*" + tag + r"\s+(\S+)\s+(\S+)\s+([0-9.eE+]+)", line)
+            if m and m.group(1) == workload and m.group(2) == kernel_key:
+                return float(m.group(3)), os.path.relpath(path, os.path.dirname(PROFILES))
+    return None, None
+
+
+# wave instructions per second all SIMDs can issue: 256 CUs x 4 SIMDs x 2.4 GHz, one VALU instruction per 4 clocks
+VALU_PEAK_GINST = 256 * 4 * 2.4 / 4.0
+
+
+def valu_issue(workload, kernel_key, kernel_ms):
+    """The march kernels are bound by VALU instruction issue, not by bytes: VALU wave instructions per launch as a
+    profiler run counted them (rocprofv3 --pmc SQ_INSTS_VALU of this script; the summary under profiles/ holds
+    the figure in a line `valu_instructions_per_launch <workload> <kernel key> <count>`) over this run's kernel
+    time, against the rate at which the chip's SIMDs can issue (no packed fp32).  A figure, not a bound to the
+    last per cent: the counter includes instructions issued with no lane active, which leave the pipe early, and the
+    clock is taken as the nominal 2.4 GHz, so a kernel at the limit can read slightly above 1.  None without such a line."""
+    count, source = _stored("valu_instructions_per_launch", workload, kernel_key)
+    if count is None or kernel_ms <= 0:
+        return None
+    rate = count / (kernel_ms * 1e-3) / 1e9
+    return dict(instructions_per_launch=count, source=source, achieved=round(rate, 1), peak=round(VALU_PEAK_GINST, 1),
+                unit="G wave instructions/s", frac=round(rate / VALU_PEAK_GINST, 4))
+
+
 def stored_traffic(workload, kernel_key):
     """HBM bytes per launch of a march kernel as a profiler run measured them: rocprofv3 --pmc FETCH_SIZE /
     WRITE_SIZE of this script, scaled by the same counters' reading for a 1 GiB copy (--calibrate-copy).
     The summary under profiles/ holds the figure in a line `traffic_bytes_per_launch <workload> <kernel key> <bytes>`;
     this run does not measure it (counters need the profiler), so the JSON line names the file it came from.
     None when there is no such line."""
-    import glob
-    import re
-    for path in sorted(glob.glob(os.path.join(PROFILES, "*.md"))):
-        for line in open(path):
-            m = re.match(r"\s*traffic_bytes_per_launch\s+(\S+)\s+(\S+)\s+([0-9.eE+]+)", line)
-            if m and m.group(1) == workload and m.group(2) == kernel_key:
-                return float(m.group(3)), os.path.relpath(path, os.path.dirname(PROFILES))
-    return None, None
+    return _stored("traffic_bytes_per_launch", workload, kernel_key)
 
 WORKLOADS = {
     # name: (scene config, n, width, height)
@@ -172,7 +195,8 @@ def inference_leg(dev, frames, warmup):
                 frame="sh + pack + march fwd, 1 view, tree built once and reused",
                 roofline=dict(bound="hbm", kernel="k_march_fwd", achieved=round(gbps, 2), peak=HBM_PEAK_GBPS, unit="GB/s",
                               frac=round(gbps / HBM_PEAK_GBPS, 5), traffic=traffic, traffic_source=source,
-                              kernel_ms=round(ms_kernel, 4), algorithmic_bytes=int(nbytes), hit_pairs_per_launch=int(hits)),
+                              kernel_ms=round(ms_kernel, 4), algorithmic_bytes=int(nbytes), hit_pairs_per_launch=int(hits),
+                              valu_issue=valu_issue(name, "march_forward", ms_kernel)),
                 frame_roofline=dict(bytes_per_frame=int(frame_bytes), frac=round(frame_bytes / (ms_frame * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
                                     roofline_fps=round(HBM_PEAK_GBPS * 1e9 / frame_bytes, 2)),
                 kernels_ms={k: round(v[0] / max(v[1], 1), 4) for k, v in timing.items() if v[1]})
@@ -372,15 +396,16 @@ def main():
     if not args.forward_only:
         cand.append(("march_backward", bwd_name, (64.0 + 56.0) * hits_per_launch + 24.0 * n_rays))
     per_kernel = {}
+    default_record = not (args.no_records or args.rec_tile_words is not None)
     for key, name, nbytes in cand:
         ms, cnt = timing[key]
         avg = ms / max(cnt, 1)
         gbps = nbytes / (avg * 1e-3) / 1e9 if avg > 0 else 0.0
         per_kernel[key] = dict(kernel=name, kernel_ms=round(avg, 4), algorithmic_bytes=int(nbytes), achieved=round(gbps, 2),
-                               frac=round(gbps / HBM_PEAK_GBPS, 5))
+                               frac=round(gbps / HBM_PEAK_GBPS, 5),
+                               valu_issue=valu_issue(args.workload, key, avg) if default_record else None)
     kname = max(per_kernel, key=lambda k: per_kernel[k]["kernel_ms"])
     dom = per_kernel[kname]
-    default_record = not (args.no_records or args.rec_tile_words is not None)
     traffic, traffic_source = stored_traffic(args.workload, kname) if default_record else (None, None)
     roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=dom["achieved"], peak=HBM_PEAK_GBPS, unit="GB/s", frac=dom["frac"],
                     traffic=traffic, traffic_source=traffic_source,

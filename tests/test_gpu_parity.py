@@ -1096,3 +1096,22 @@ def test_settings_update_refits_inside_the_render_function(gx):
     for k, a, b in zip(names, g_u, g_n):
         c, r = gx.cos_rel(a, b)
         assert c >= 0.99999 and r <= 1e-4, (k, c, r)
+
+
+@pytest.mark.gpu
+def test_scratch_of_streams_no_longer_used_is_dropped(gx, c0):
+    """The host mirror keeps one set of scratch tensors per stream in use; a loop that keeps making new
+    streams must not keep a set for each of them."""
+    from raygaussx_amd import optix_utils as u_ox
+    scene, cam, cfg = c0
+    small = scenes.make_camera(0, 0, width=32, height=24)
+    want = gx.gpu_render(scene, small, cfg, stats=False)["image"]
+    for _ in range(2 * u_ox._SCRATCH_STREAMS + 3):
+        s = torch.cuda.Stream()
+        with torch.cuda.stream(s):
+            got = gx.gpu_render(scene, small, cfg, stats=False)["image"]
+        assert np.array_equal(got, want)
+    per_key = {}
+    for key, dev, _stream in u_ox._scratch:
+        per_key[(key, dev)] = per_key.get((key, dev), 0) + 1
+    assert per_key and max(per_key.values()) <= u_ox._SCRATCH_STREAMS

@@ -906,6 +906,16 @@ __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, 
 template <int H>
 struct Half {
     static constexpr int value = H;
+    static constexpr int group = 16; // lanes that share a trip's entry: a row
+};
+// Tag of a walk in which the two halves of a row (8 lanes each) walk on their own.  (Groups of 4 make
+// still fewer trips, but four times a row's adds to the window's sums in LDS: measured slower.)
+#ifndef RGX_GRAD_GROUP
+#define RGX_GRAD_GROUP 8
+#endif
+struct HalfRows {
+    static constexpr int value = 0;
+    static constexpr int group = RGX_GRAD_GROUP;
 };
 
 // Shade: the four rows walk their own lists in lock step; body(entry, hit, live) runs whenever
@@ -1253,17 +1263,48 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
             __syncthreads();
             slots = RL.rowlist + row * RGX_CCAP;
         }
-        uint32_t bits = 0;
-        for (int i = 0; i < maxlen; ++i) {
-            if ((i & 31) == 0) bits = masks[(i >> 5) * 64];
-            const bool live = i < len;
-            const bool hit = run && live && ((bits >> (i & 31)) & 1u);
-            if (COUNT && hit) ++p0;
-            if (__ballot(hit)) {
-                const int slot = live ? min((int)slots[min(i, RGX_CCAP - 1)], RGX_CCAP - 1) : 0;
-                const int32_t pid = (int32_t)(RL.pid[slot] & ~RGX_SLOT_TOUCHED);
-                body(Entry<false>{(const float4 *)(RL.frame + slot), P.prims + pid, pid, slot}, hit, live, Half<0>{});
+        static_assert(!COUNT, "the rows' walk counts nothing");
+        (void)maxlen;
+        // Each half of a row (8 lanes, 2 x 4 pixels) walks the entries that one of its own rays hits: the set bits
+        // of the OR of its lanes' masks.  Fewer trips than with whole rows in lock step (a trip lasts until the
+        // longest list of the wave is done, and half a row's list is shorter than the row's).
+        const int nwr = min((len + 31) >> 5, nw);
+        auto lane_word = [&](int w) {
+            const int left = len - w * 32;
+            return (run ? masks[w * 64] : 0u) & (left >= 32 ? ~0u : ((1u << left) - 1u));
+        };
+        auto group_or = [](uint32_t m) {
+            m |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
+            m |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x4E, 0xf, 0xf, true);  // quad_perm [2,3,0,1]
+            if (RGX_GRAD_GROUP >= 8) m |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0x141, 0xf, 0xf, true); // row_half_mirror
+            return m;
+        };
+        int w = 0;
+        uint32_t mword = nwr > 0 ? lane_word(0) : 0u;
+        uint32_t bits = group_or(mword);
+        for (;;) {
+            // (all lanes of a group hold the same bits and the same w: the DPP moves below run with the whole group active)
+            while (__any(bits == 0u && w + 1 < nwr)) {
+                const bool next = bits == 0u && w + 1 < nwr;
+                const uint32_t m = next ? lane_word(w + 1) : 0u;
+                const uint32_t o = group_or(m);
+                if (next) {
+                    ++w;
+                    mword = m;
+                    bits = o;
+                }
             }
+            const bool live = bits != 0u;
+            if (!__any(live)) break;
+            int pos = 0;
+            if (live) {
+                pos = __builtin_ctz(bits);
+                bits &= bits - 1u;
+            }
+            const bool hit = live && ((mword >> pos) & 1u);
+            const int slot = live ? min((int)slots[min(w * 32 + pos, RGX_CCAP - 1)], RGX_CCAP - 1) : 0;
+            const int32_t pid = (int32_t)(RL.pid[slot] & ~RGX_SLOT_TOUCHED);
+            body(Entry<false>{(const float4 *)(RL.frame + slot), P.prims + pid, pid, slot}, hit, live, HalfRows{});
         }
     }
     return 8 + q0 + q1 + q2 + q3 + nw * 72;
@@ -1704,12 +1745,13 @@ __device__ __forceinline__ float row_take(float v)
 {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float row_sum(float v)
+template <int GROUP>
+__device__ __forceinline__ float group_sum(float v)
 {
     v += row_take<0xB1>(v);  // quad_perm [1,0,3,2]
     v += row_take<0x4E>(v);  // quad_perm [2,3,0,1]
-    v += row_take<0x141>(v); // row_half_mirror
-    v += row_take<0x140>(v); // row_mirror
+    if constexpr (GROUP >= 8) v += row_take<0x141>(v); // row_half_mirror
+    if constexpr (GROUP == 16) v += row_take<0x140>(v); // row_mirror
     return v;
 }
 
@@ -1852,7 +1894,8 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                 return has;
             };
             // (3) per table entry: moments per lane, row sum, one set of atomics per row
-            auto gradients = [&](const auto &e, bool hit, bool live, auto) {
+            auto gradients = [&](const auto &e, bool hit, bool live, auto which) {
+                constexpr int GROUP = decltype(which)::group; // lanes that share this trip's entry
                 float out[RGX_NSUM];
 #pragma unroll
                 for (int c = 0; c < RGX_NSUM; ++c) out[c] = 0.f;
@@ -1900,11 +1943,11 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                     out[11] = fmaf(Mxc.x, B.z, Md.x * E.z);
                     out[12] = fmaf(Mxc.y, B.z, Md.y * E.z);
                 }
-                // summed over the row's rays; one lane per row carries the sums on
+                // summed over the group's rays; one lane per group carries the sums on
                 const uint64_t bal = __ballot(hit);
 #pragma unroll
-                for (int c = 0; c < RGX_NSUM; ++c) out[c] = row_sum(out[c]);
-                if ((lane & 15) == 0 && live && ((bal >> lane) & 0xffffull)) {
+                for (int c = 0; c < RGX_NSUM; ++c) out[c] = group_sum<GROUP>(out[c]);
+                if ((lane & (GROUP - 1)) == 0 && live && ((bal >> lane) & ((1ull << GROUP) - 1ull))) {
                     if constexpr (REPLAY) {
                         // to the window's sums in LDS; a slot's first touch is what replay_flush()
                         // later turns into 14 adds to memory

@@ -837,13 +837,18 @@ struct LaneQuery {
 // not counted again.  PLAIN: every entry of the table passed plain_roots().
 template <bool SEARCH, int PART, bool PLAIN, typename Cn>
 __device__ __forceinline__ void filter_table(const TileLds &L, int C, float t0, float t1, const LaneQuery &Q, int &p0, bool &ov,
-                                             float &found, int &len, Cn &cn)
+                                             float &found, int &len, uint32_t (&own)[2], Cn &cn)
 {
     const int lane = threadIdx.x, row = lane >> 4;
     len = 0;
+    own[0] = own[1] = 0u;
     uint32_t bits = 0, first = 0, second = 0; // this lane's hits; those with samples in the first / second half
     auto flush = [&](int w) {
         L.mask[w][lane] = bits;
+        if (w == 0) { // the ray's own notes on the list's first 32 entries stay with it (see shade_lanes)
+            own[0] = first;
+            own[1] = second;
+        }
         const uint32_t f = row_or(first), g = row_or(second);
         if ((lane & 15) == 0) {
             L.half[0][row][w] = f;
@@ -945,14 +950,17 @@ __device__ __forceinline__ void shade_rows(const MarchParams &P, const TileLds &
 // row's list), so the trip count is the longest hit list of a ray instead of the longest row list.
 // For bodies that need no sum over the rays of a row.  The order of a ray's hits is that of
 // shade_rows.  Only the entries that can reach half `half` of the slab's samples are visited; the
-// body gets Half<TAG>.
+// body gets Half<TAG>.  For the list's first 32 entries the ray goes by its own chords (own[half]: its
+// hits with samples in that half, as the filter left them), for the rest by its row's notes, which
+// also hold for rays whose own chord stays in the other half.
 template <int TAG, typename Body>
-__device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds &L, int len, bool run, int half, Body body)
+__device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds &L, int len, bool run, int half,
+                                            const uint32_t (&own)[2], Body body)
 {
     const int lane = threadIdx.x, row = lane >> 4;
     const int nw = (len + 31) >> 5;
     int w = 0;
-    uint32_t bits = (run && nw > 0) ? L.mask[0][lane] & L.half[half][row][0] : 0u;
+    uint32_t bits = (run && nw > 0) ? (half ? own[1] : own[0]) : 0u;
     for (;;) {
         while (bits == 0u && run && w + 1 < nw) {
             ++w;
@@ -1356,6 +1364,7 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
     // phase 1 those that reach the second 16, and a Gaussian of both halves is counted once.
     const bool split = WALK == WALK_FORWARD && std::is_same<Rec, NoRecorder>::value && Wn.crowded && __any(need);
     int len = 0, q0 = 0, seen = 0;
+    uint32_t own[2] = {0u, 0u}; // this ray's hits among the list's first 32 entries, by half of the samples
     bool run = need, qov = false;
     for (int phase = 0; phase < 2; ++phase) {
         const bool reuse = !split && Wn.resident && t1 <= Wn.hi;
@@ -1419,8 +1428,8 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                 float best = phase == 0 ? found : -1.0f;
                 auto filter = [&](auto search, auto part) {
                     const float far = decltype(search)::value ? cover : hi;
-                    if (std::is_same<Rec, NoRecorder>::value ? __builtin_expect(plain, 1) : plain) filter_table<decltype(search)::value, decltype(part)::value, true>(L, C, lo, far, Q, cnt, cut, best, len, cn);
-                    else filter_table<decltype(search)::value, decltype(part)::value, false>(L, C, lo, far, Q, cnt, cut, best, len, cn);
+                    if (std::is_same<Rec, NoRecorder>::value ? __builtin_expect(plain, 1) : plain) filter_table<decltype(search)::value, decltype(part)::value, true>(L, C, lo, far, Q, cnt, cut, best, len, own, cn);
+                    else filter_table<decltype(search)::value, decltype(part)::value, false>(L, C, lo, far, Q, cnt, cut, best, len, own, cn);
                 };
                 using std::integral_constant;
                 if (!split) {
@@ -1447,11 +1456,11 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
             }
             if constexpr (WALK == WALK_FORWARD) {
                 static_assert(std::is_same<BodyA, BodyB>::value, "the forward shades both halves with one body");
-                shade_lanes<0>(P, L, len, run, phase, body_a);
+                shade_lanes<0>(P, L, len, run, phase, own, body_a);
             } else if constexpr (WALK == WALK_BACKWARD) {
                 if (phase == 0) {
-                    shade_lanes<0>(P, L, len, run, 0, body_a);
-                    shade_lanes<1>(P, L, len, run, 1, body_a);
+                    shade_lanes<0>(P, L, len, run, 0, own, body_a);
+                    shade_lanes<1>(P, L, len, run, 1, own, body_a);
                 } else {
                     shade_rows(P, L, len, run, body_b);
                 }

@@ -153,3 +153,20 @@ def test_record_size_fits_a_memory_budget():
     assert u_ox.fit_tile_words(cs, u_ox.REC_TILE_WORDS, 10 * 2**30) == u_ox.REC_LIST_WORDS
     assert u_ox.fit_tile_words(cs, u_ox.REC_TILE_WORDS, 2**30) == 0
     assert u_ox.fit_tile_words(cs, 4096, 10 * 2**30) == 4096     # a caller's small record is left alone
+
+
+def test_bench_finds_its_stored_profile_figures():
+    """bench.py reports HBM traffic and VALU instructions per launch from the summaries under profiles/ (a run
+    without the profiler cannot count them): the lines it looks for are there, for both timed workloads."""
+    import importlib.util
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..")
+    spec = importlib.util.spec_from_file_location("bench_for_test", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    for workload, key in (("c4_1M_800x800", "march_forward"), ("c4_1M_800x800", "march_backward"),
+                          ("c3_3M_1920x1080_fwd", "march_forward")):
+        traffic, source = bench.stored_traffic(workload, key)
+        assert traffic and traffic > 1e8 and source.startswith("profiles/") and os.path.exists(os.path.join(root, source))
+        issue = bench.valu_issue(workload, key, 7.0)
+        assert issue and issue["instructions_per_launch"] > 1e9 and 0.0 < issue["frac"] < 4.0
+    assert bench.stored_traffic("c4_1M_800x800", "no_such_kernel") == (None, None)

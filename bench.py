@@ -23,9 +23,18 @@ reaches on this GPU (read + written bytes), the practical ceiling beside the 8 T
 Beside the contract's keys: ``atomics`` (the gradient scatter's atomic adds per backward launch,
 counted by the kernels, over the launch's time) and ``views_in_flight`` (the same steps timed once
 more with two views in flight on two streams, as a loop that accumulates gradients over several
-views can run them; ``value`` itself is always one view at a time).
+views can run them; ``value`` itself is always one view at a time).  ``other_workloads``: the other
+benchmark configurations (300 k Gaussians at 800x800, 3 M at 1237x822, 1 M at 1024x1024), five steps each,
+with their own step and kernel rooflines.  ``valu_measured``: the rate at which this card issues VALU
+instructions, from a kernel of independent multiply-adds run here; it is the ``peak`` of every
+``valu_issue`` figure (whose instruction counts are stored figures of a profiler run, see ``valu_issue``).
+``--workload coherent_512_800x800`` is not a benchmark configuration but the kernels' best case (every ray
+of a tile hits the same few large Gaussians for whole slabs); ``--sections`` reads the per-section cycle
+census of a diagnostic build of the library (``python -m raygaussx_amd.build --sections``, selected with
+``RGX_LIB_PATH``).
 """
 import argparse
+import ctypes as C
 import json
 import os
 import sys
@@ -58,23 +67,52 @@ def _stored(tag, workload, kernel_key):
     return None, None
 
 
-# wave instructions per second all SIMDs can issue: 256 CUs x 4 SIMDs x 2.4 GHz, one VALU instruction per 4 clocks
-VALU_PEAK_GINST = 256 * 4 * 2.4 / 4.0
+# wave instructions per second all SIMDs could issue at the nominal clock: 256 CUs x 4 SIMDs x 2.4 GHz, one VALU
+# instruction per 4 clocks.  Reported beside the measured rate; the measured rate is the one fractions are taken of.
+VALU_NOMINAL_GINST = 256 * 4 * 2.4 / 4.0
+_valu_measured = None
 
 
-def valu_issue(workload, kernel_key, kernel_ms):
-    """The march kernels are bound by VALU instruction issue, not by bytes: VALU wave instructions per launch as a
-    profiler run counted them (rocprofv3 --pmc SQ_INSTS_VALU of this script; the summary under profiles/ holds
-    the figure in a line `valu_instructions_per_launch <workload> <kernel key> <count>`) over this run's kernel
-    time, against the rate at which the chip's SIMDs can issue (no packed fp32).  A figure, not a bound to the
-    last per cent: the counter includes instructions issued with no lane active, which leave the pipe early, and the
-    clock is taken as the nominal 2.4 GHz, so a kernel at the limit can read slightly above 1.  None without such a line."""
+def valu_measured(dev):
+    """G VALU wave instructions per second this card issues, measured: a kernel of independent fp32
+    multiply-adds (rgx_probe_valu_rate: 8 wavefronts per SIMD, nothing but v_fma_f32 and a loop counter), its
+    instruction count known from its shape, timed with events on the launch stream; best of five launches."""
+    global _valu_measured
+    if _valu_measured is None:
+        sink = torch.zeros(4, device=dev)
+        count = C.c_uint64(0)
+        waves, iters = 256 * 4 * 8, 2048
+        best = float("inf")
+        for rep in range(7):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            L.check(L.lib().rgx_probe_valu_rate(C.c_int32(waves), C.c_int32(iters), L.ptr(sink), C.byref(count), L.stream(dev)))
+            b.record()
+            torch.cuda.synchronize()
+            if rep >= 2:
+                best = min(best, a.elapsed_time(b))
+        _valu_measured = dict(value=round(count.value / (best * 1e-3) / 1e9, 1), unit="G wave instructions/s",
+                              nominal=round(VALU_NOMINAL_GINST, 1), instructions=count.value, kernel_ms=round(best, 4),
+                              what="independent v_fma_f32 chains, 8 wavefronts per SIMD")
+    return _valu_measured
+
+
+def valu_issue(workload, kernel_key, kernel_ms, dev):
+    """The march kernels are bound by VALU instruction issue, not by bytes.  ``instructions_per_launch`` is a STORED
+    figure: VALU wave instructions per launch as a profiler run of this script counted them (rocprofv3 --pmc
+    SQ_INSTS_VALU; the summary under profiles/ holds it in a line `valu_instructions_per_launch <workload> <kernel
+    key> <count>`), divided by THIS run's kernel time; ``peak`` is the issue rate measured on this card in this run
+    (``valu_measured``).  The stored count and this run's time belong to different launches of the same
+    deterministic kernel on the same inputs; should the pairing ever read above the measured peak it is reported as
+    such (``above_peak``) and ``frac`` is capped at 1.  None without a stored line."""
     count, source = _stored("valu_instructions_per_launch", workload, kernel_key)
     if count is None or kernel_ms <= 0:
         return None
+    peak = valu_measured(dev)["value"]
     rate = count / (kernel_ms * 1e-3) / 1e9
-    return dict(instructions_per_launch=count, source=source, achieved=round(rate, 1), peak=round(VALU_PEAK_GINST, 1),
-                unit="G wave instructions/s", frac=round(rate / VALU_PEAK_GINST, 4))
+    return dict(instructions_per_launch=count, count_is="stored (profiler run)", source=source, achieved=round(rate, 1),
+                peak=peak, peak_is="measured in this run", unit="G wave instructions/s", frac=round(min(rate / peak, 1.0), 4),
+                above_peak=bool(rate > peak))
 
 
 def stored_traffic(workload, kernel_key):
@@ -92,6 +130,8 @@ WORKLOADS = {
     "c4_1M_1024x1024": (4, 1_000_000, 1024, 1024),
     "c2_3M_1237x822": (2, 3_000_000, 1237, 822),
     "c0_4096_128x128": (0, 4096, 128, 128),
+    # not a benchmark configuration: the kernels' best case (see scenes.CONFIGS["coherent"])
+    "coherent_512_800x800": ("coherent", 512, 800, 800),
     # inference along a camera path, tree built once (scripts/test.py:60-126): frames per second
     "c3_3M_1920x1080_fwd": (3, 3_000_000, 1920, 1080),
 }
@@ -196,7 +236,7 @@ def inference_leg(dev, frames, warmup):
                 roofline=dict(bound="hbm", kernel="k_march_fwd", achieved=round(gbps, 2), peak=HBM_PEAK_GBPS, unit="GB/s",
                               frac=round(gbps / HBM_PEAK_GBPS, 5), traffic=traffic, traffic_source=source,
                               kernel_ms=round(ms_kernel, 4), algorithmic_bytes=int(nbytes), hit_pairs_per_launch=int(hits),
-                              valu_issue=valu_issue(name, "march_forward", ms_kernel)),
+                              valu_issue=valu_issue(name, "march_forward", ms_kernel, dev)),
                 frame_roofline=dict(bytes_per_frame=int(frame_bytes), frac=round(frame_bytes / (ms_frame * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
                                     roofline_fps=round(HBM_PEAK_GBPS * 1e9 / frame_bytes, 2)),
                 kernels_ms={k: round(v[0] / max(v[1], 1), 4) for k, v in timing.items() if v[1]})
@@ -256,56 +296,41 @@ def side_kernels(dev, reps):
     return dict(side_kernels=out, reps=reps, data="synthetic")
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c4_1M_800x800", choices=sorted(WORKLOADS))
-    ap.add_argument("--cpu-rays", type=int, default=262144, help="ray sample of the CPU baseline (0 = skip)")
-    ap.add_argument("--fps-frames", type=int, default=20,
-                    help="after the headline pass, frames of the 3 M-Gaussian 1920x1080 forward-only orbit to time for "
-                         "`fwd_fps_c3` (0 = skip; skipped for workloads other than the default)")
-    ap.add_argument("--forward-only", action="store_true")
-    ap.add_argument("--no-records", action="store_true",
-                    help="backward searches the tree again instead of replaying the forward's hit-list record")
-    ap.add_argument("--rec-tile-words", type=int, default=None,
-                    help="record size per tile in 32-bit words (16384: hit lists only, no per-sample sums); "
-                         "default: the renderer's own")
-    ap.add_argument("--in-flight", type=int, default=2,
-                    help="after the timed steps, time the same steps again with this many views in flight, each on "
-                         "a stream of its own (reported beside the headline figure; 1 = skip)")
-    ap.add_argument("--side-kernels", action="store_true",
-                    help="time the entry points around the march (image epilogue, reorder gather, distCUDA2, viewer launch) "
-                         "instead of the training step; one JSON line")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="only run a 1 GiB device-to-device copy (reference reading for the FETCH_SIZE / WRITE_SIZE counters)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU only (--gpus 1); the path would shard by views or bands "
-                 "of tiles with one gradient all-reduce per step, but no multi-GPU figure is produced")
-    if not torch.cuda.is_available():
-        sys.exit("bench.py: needs a GPU (librgx has no CPU path)")
-    dev = "cuda:0"
-    if args.calibrate_copy:
-        src = torch.full((1 << 28,), 1.0, dtype=torch.float32, device=dev)     # 1 GiB
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        print(json.dumps(dict(calibration="copy", bytes_read=src.numel() * 4, bytes_written=dst.numel() * 4, launches=3)))
-        return
-    L.lib()
-    if args.side_kernels:
-        print(json.dumps(side_kernels(dev, args.steps)), flush=True)
-        return
-    config, n, width, height = WORKLOADS[args.workload]
+SECTION_NAMES = ("sweep", "filter", "shade_or_gradient_trips", "record_lists", "blend_or_prefix", "sample_sums_io",
+                 "tile_setup", "iteration_top", "iteration_end", "epilogue", "walk_and_parse", "flush_gradients")
+SECTION_KERNELS = ("k_march_fwd<record>", "k_march_fwd<plain>", "k_march_bwd_replay_sums", "k_march_bwd_replay", "k_march_bwd")
+
+
+def read_sections(reset=False):
+    """The per-section cycle census of a diagnostic build (python -m raygaussx_amd.build --sections): per march kernel
+    the share of its waves' lifetimes spent in each section, or None when the loaded library has no census."""
+    lib = L.lib()
+    if not hasattr(lib, "rgx_debug_section_cycles"):
+        return None
+    nsec = len(SECTION_NAMES)
+    raw = (C.c_uint64 * (len(SECTION_KERNELS) * (nsec + 1)))()
+    L.check(lib.rgx_debug_section_cycles(raw, int(reset)))
+    out = {}
+    for k, kernel in enumerate(SECTION_KERNELS):
+        row = [int(raw[k * (nsec + 1) + i]) for i in range(nsec + 1)]
+        total = sum(row[:nsec])
+        if row[nsec] and total:
+            out[kernel] = dict(waves=row[nsec], cycles_per_wave=round(total / row[nsec]),
+                               shares={name: round(c / total, 4) for name, c in zip(SECTION_NAMES, row[:nsec]) if c})
+    return out
+
+
+def training_leg(dev, workload, steps, warmup, opts, in_flight=1):
+    """``steps`` timed training steps (or frames) of one workload; returns (JSON fields, the CPU scene, cfg)."""
+    config, n, width, height = WORKLOADS[workload]
     cfg = dict(scenes.CONFIGS[config])
     scene = scenes.make_scene(config, n=n)
     dscene = {k: v.to(dev) for k, v in scene.items()}
     names = ("positions", "scales", "quaternions", "densities", "color_features", "sph_gauss_features",
              "bandwidth_sharpness", "lobe_axis")
-    params = [dscene[k].clone().requires_grad_(not args.forward_only) for k in names]
+    inference = workload.endswith("_fwd")
+    forward_only = opts.forward_only or inference
+    params = [dscene[k].clone().requires_grad_(not forward_only) for k in names]
     n_cams = min(cfg["n_cameras"], 100)
     cams = [scenes.make_camera(config, i, width=width, height=height).to(dev) for i in range(n_cams)]
     cam_structs = [u_ox.camera_struct(c) for c in cams]   # also caches each camera's host constants: no sync per step
@@ -313,9 +338,7 @@ def main():
     target = torch.rand(n_rays, 3, device=dev, generator=torch.Generator(dev).manual_seed(1))
     stats = u_ox.new_stats(dev)
     gas = None
-    inference = args.workload.endswith("_fwd")
     if inference:
-        args.forward_only = True
         from raygaussx_amd.render_optix import compute_rgb
         tree = u_ox.AccelerationStructure(n, dev).build_from_gaussians(dscene["positions"], dscene["scales"],
                                                                         dscene["quaternions"], dscene["densities"])
@@ -341,120 +364,224 @@ def main():
         s = default_settings(cams[i % n_cams], cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
                              t_eps=cfg["t_eps"], gas=gas)
         s.stats = stats if census else None
-        s.record_hits = not args.no_records
-        if args.rec_tile_words is not None:
-            s.rec_tile_words = args.rec_tile_words
+        s.record_hits = not opts.no_records
+        if opts.rec_tile_words is not None:
+            s.rec_tile_words = opts.rec_tile_words
         img = RenderOptixFunction.apply(*params, s)
         gas = s.gas
-        if not args.forward_only:
+        if not forward_only:
             loss = ((img - target) ** 2).mean()
             loss.backward()
             for p in params:
                 p.grad = None
         return img
 
-    for i in range(args.warmup):
+    torch.cuda.reset_peak_memory_stats(dev)
+    base_mem = torch.cuda.memory_allocated(dev)
+    step(0)                        # the first view of a shape: its record is sized before anything is known of its use
+    torch.cuda.synchronize()
+    first_peak = torch.cuda.max_memory_allocated(dev)
+    for i in range(1, warmup):
         step(i)
     torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats(dev)
+    if opts.sections:
+        read_sections(reset=True)
     L.timing_enable(True)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for i in range(args.steps):
-        step(args.warmup + i)
+    for i in range(steps):
+        step(warmup + i)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     timing = L.timing_read()
     L.timing_enable(False)
-    for i in range(args.steps):     # census: the same views once more, counted, not timed
-        step(args.warmup + i, census=True)
+    sections = read_sections() if opts.sections else None
+    steady_peak = torch.cuda.max_memory_allocated(dev)
+    for i in range(steps):     # census: the same views once more, counted, not timed
+        step(warmup + i, census=True)
     torch.cuda.synchronize()
     st = u_ox.read_stats(stats)
-    in_flight = None
-    if args.in_flight > 1:     # views of one accumulation window are independent: keep several in flight
-        lanes = [(torch.cuda.Stream(dev), [None]) for _ in range(args.in_flight)]
-        for i in range(max(args.warmup, args.in_flight)):
+    flight = None
+    if in_flight > 1:     # views of one accumulation window are independent: keep several in flight
+        lanes = [(torch.cuda.Stream(dev), [None]) for _ in range(in_flight)]
+        for i in range(max(warmup, in_flight)):
             step(i, lane=lanes[i % len(lanes)])
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(args.steps):
-            step(args.warmup + i, lane=lanes[i % len(lanes)])
+        for i in range(steps):
+            step(warmup + i, lane=lanes[i % len(lanes)])
         torch.cuda.synchronize()
         el = time.perf_counter() - t0
-        in_flight = dict(views=args.in_flight, value=round(n_rays * args.steps / el / 1e6, 4), unit="Mrays/s",
-                         ms_per_step=round(el / args.steps * 1e3, 4))
+        flight = dict(views=in_flight, value=round(n_rays * steps / el / 1e6, 4), unit="Mrays/s",
+                      ms_per_step=round(el / steps * 1e3, 4))
         if inference:
-            in_flight["frames_per_s"] = round(args.steps / el, 3)
+            flight["frames_per_s"] = round(steps / el, 3)
 
-    ms_per_step = elapsed / args.steps * 1e3
-    mrays = n_rays * args.steps / elapsed / 1e6
-    passes = 1 if args.forward_only else 2
-    hits_per_launch = st["hit_pairs"] / (args.steps * passes)   # H: fwd and bwd march the same slabs
+    ms_per_step = elapsed / steps * 1e3
+    mrays = n_rays * steps / elapsed / 1e6
+    passes = 1 if forward_only else 2
+    hits_per_launch = st["hit_pairs"] / (steps * passes)   # H: fwd and bwd march the same slabs
     # the dominant kernel: the march launch (forward or backward) that takes longer
-    bwd_name = "k_march_bwd" if args.no_records else (
-        "k_march_bwd_replay" if (args.rec_tile_words or 1 << 30) < 16384 + 8192 else "k_march_bwd_replay_sums")
+    bwd_name = "k_march_bwd" if opts.no_records else (
+        "k_march_bwd_replay" if (opts.rec_tile_words or 1 << 30) < 16384 + 8192 else "k_march_bwd_replay_sums")
     cand = [("march_forward", "k_march_fwd", 64.0 * hits_per_launch + 12.0 * n_rays)]
-    if not args.forward_only:
+    if not forward_only:
         cand.append(("march_backward", bwd_name, (64.0 + 56.0) * hits_per_launch + 24.0 * n_rays))
     per_kernel = {}
-    default_record = not (args.no_records or args.rec_tile_words is not None)
+    default_record = not (opts.no_records or opts.rec_tile_words is not None)
     for key, name, nbytes in cand:
         ms, cnt = timing[key]
         avg = ms / max(cnt, 1)
         gbps = nbytes / (avg * 1e-3) / 1e9 if avg > 0 else 0.0
         per_kernel[key] = dict(kernel=name, kernel_ms=round(avg, 4), algorithmic_bytes=int(nbytes), achieved=round(gbps, 2),
                                frac=round(gbps / HBM_PEAK_GBPS, 5),
-                               valu_issue=valu_issue(args.workload, key, avg) if default_record else None)
+                               valu_issue=valu_issue(workload, key, avg, dev) if default_record else None)
     kname = max(per_kernel, key=lambda k: per_kernel[k]["kernel_ms"])
     dom = per_kernel[kname]
-    traffic, traffic_source = stored_traffic(args.workload, kname) if default_record else (None, None)
+    traffic, traffic_source = stored_traffic(workload, kname) if default_record else (None, None)
     roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=dom["achieved"], peak=HBM_PEAK_GBPS, unit="GB/s", frac=dom["frac"],
                     traffic=traffic, traffic_source=traffic_source,
                     kernel_ms=dom["kernel_ms"], algorithmic_bytes=dom["algorithmic_bytes"],
                     hit_pairs_per_launch=int(hits_per_launch), march_kernels=per_kernel)
     # whole-step roofline-derived rate: all algorithmic bytes of one step at peak bandwidth
     step_bytes = (64.0 * hits_per_launch + 12.0 * n_rays + 300.0 * n
-                  + (0 if args.forward_only else (120.0 * hits_per_launch + 24.0 * n_rays + 464.0 * n)))
-    out = dict(metric="Mrays/s fwd" + ("" if args.forward_only else "+bwd"), value=round(mrays, 4), unit="Mrays/s",
-               n_gpus=1, steps=args.steps, warmup=args.warmup, ms_per_step=round(ms_per_step, 4),
+                  + (0 if forward_only else (120.0 * hits_per_launch + 24.0 * n_rays + 464.0 * n)))
+    out = dict(metric="Mrays/s fwd" + ("" if forward_only else "+bwd"), value=round(mrays, 4), unit="Mrays/s",
+               n_gpus=1, steps=steps, warmup=warmup, ms_per_step=round(ms_per_step, 4),
                higher_is_better=True, scaling="weak", vs_baseline=None, dtype="f32", data="synthetic",
-               config=dict(workload=args.workload, gaussians=n, width=width, height=height, sh_degree=3,
+               config=dict(workload=workload, gaussians=n, width=width, height=height, sh_degree=3,
                            dt_step=cfg["dt_step"], dynamic_sampling=cfg["dynamic_sampling"],
                            max_prim_slice=cfg["max_prim_slice"], t_eps=cfg["t_eps"],
                            step=("sh + pack + march fwd, 1 view, tree built once" if inference else
                                  "bvh build + sh + pack + march fwd"
-                                 + ("" if args.forward_only else " + march bwd + sh bwd") + ", 1 view")),
+                                 + ("" if forward_only else " + march bwd + sh bwd") + ", 1 view")),
                roofline=roofline,
                step_roofline=dict(bytes_per_step=int(step_bytes),
                                   achieved=round(step_bytes / (ms_per_step * 1e-3) / 1e9, 2), unit="GB/s",
                                   frac=round(step_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 5),
                                   roofline_mrays=round(HBM_PEAK_GBPS * 1e9 * n_rays / step_bytes / 1e6, 2)),
                kernels_ms={k: round(v[0] / max(v[1], 1), 4) for k, v in timing.items() if v[1]},
-               stats_per_step={k: v / args.steps for k, v in st.items()})
+               stats_per_step={k: v / steps for k, v in st.items()})
     if inference:
         out["frames_per_s"] = round(1e3 / ms_per_step, 3)
-    if not args.forward_only:   # the gradient scatter: fp32 atomic adds to memory per backward launch (census) over its time
-        adds = st["grad_atomics"] / args.steps
+    if not forward_only:   # the gradient scatter: fp32 atomic adds to memory per backward launch (census) over its time
+        adds = st["grad_atomics"] / steps
         out["atomics"] = dict(per_backward_launch=int(adds), unit="G atomic adds/s",
                               value=round(adds / (per_kernel["march_backward"]["kernel_ms"] * 1e-3) / 1e9, 3))
-    out["views_in_flight"] = in_flight
-    rec_use = None if (inference or args.forward_only) else u_ox.record_use(cam_structs[0], dev)
-    out["memory"] = dict(peak_allocated_GB=round(torch.cuda.max_memory_allocated(dev) / 1e9, 3),
+    # lane-slots per ray-slab-hit pair from this run's kernel time: what the launch could have issued at the measured
+    # VALU rate, per pair -- an upper bound of the instructions actually issued (the profiler's count is in valu_issue)
+    rate = valu_measured(dev)["value"] * 1e9
+    for key in per_kernel:
+        per_kernel[key]["lane_slots_per_pair_at_measured_issue_rate"] = (
+            round(per_kernel[key]["kernel_ms"] * 1e-3 * rate * 64.0 / hits_per_launch, 1) if hits_per_launch else None)
+    out["views_in_flight"] = flight
+    if sections is not None:
+        out["sections"] = sections
+    rec_use = None if forward_only else u_ox.record_use(cam_structs[0], dev, n)
+    out["memory"] = dict(first_view_peak_GB=round(first_peak / 1e9, 3), steady_peak_GB=round(steady_peak / 1e9, 3),
+                         first_over_steady=round(first_peak / max(steady_peak, 1), 3),
+                         resident_before_GB=round(base_mem / 1e9, 3),
                          record_allocated_GB=None if rec_use is None else round(rec_use[0] / 1e9, 3),
                          record_used_GB=None if rec_use is None else round(rec_use[1] / 1e9, 3))
-    del params, dscene, target
+    del params, dscene, target, stats
     gas = None
     torch.cuda.empty_cache()
+    return out, scene, cfg
+
+
+OTHER_WORKLOADS = ("c1_300k_800x800", "c2_3M_1237x822", "c4_1M_1024x1024")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c4_1M_800x800", choices=sorted(WORKLOADS))
+    ap.add_argument("--cpu-rays", type=int, default=262144, help="ray sample of the CPU baseline (0 = skip)")
+    ap.add_argument("--fps-frames", type=int, default=20,
+                    help="after the headline pass, frames of the 3 M-Gaussian 1920x1080 forward-only orbit to time for "
+                         "`fwd_fps_c3` (0 = skip; skipped for workloads other than the default)")
+    ap.add_argument("--other-steps", type=int, default=5,
+                    help="after the headline pass, timed steps of each other benchmark configuration for `other_workloads` "
+                         "(0 = skip; skipped for workloads other than the default)")
+    ap.add_argument("--forward-only", action="store_true")
+    ap.add_argument("--no-records", action="store_true",
+                    help="backward searches the tree again instead of replaying the forward's hit-list record")
+    ap.add_argument("--rec-tile-words", type=int, default=None,
+                    help="record size per tile in 32-bit words (16384: hit lists only, no per-sample sums); "
+                         "default: the renderer's own")
+    ap.add_argument("--in-flight", type=int, default=2,
+                    help="after the timed steps, time the same steps again with this many views in flight, each on "
+                         "a stream of its own (reported beside the headline figure; 1 = skip)")
+    ap.add_argument("--sections", action="store_true",
+                    help="also report the march kernels' per-section cycle census; needs the diagnostic build "
+                         "(python -m raygaussx_amd.build --sections; RGX_LIB_PATH=raygaussx_amd/librgx_sections.so)")
+    ap.add_argument("--side-kernels", action="store_true",
+                    help="time the entry points around the march (image epilogue, reorder gather, distCUDA2, viewer launch) "
+                         "instead of the training step; one JSON line")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a 1 GiB device-to-device copy (reference reading for the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--calibrate-valu", action="store_true",
+                    help="only run the multiply-add kernel of `valu_measured` (reference reading for the SQ_INSTS_VALU counter)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (--gpus 1); the path would shard by views or bands "
+                 "of tiles with one gradient all-reduce per step, but no multi-GPU figure is produced")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: needs a GPU (librgx has no CPU path)")
+    dev = "cuda:0"
+    if args.calibrate_copy:
+        src = torch.full((1 << 28,), 1.0, dtype=torch.float32, device=dev)     # 1 GiB
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps(dict(calibration="copy", bytes_read=src.numel() * 4, bytes_written=dst.numel() * 4, launches=3)))
+        return
+    L.lib()
+    if args.calibrate_valu:
+        print(json.dumps(dict(calibration="valu", launches=7, **valu_measured(dev))))
+        return
+    if args.side_kernels:
+        print(json.dumps(side_kernels(dev, args.steps)), flush=True)
+        return
+    if args.sections and read_sections() is None:
+        sys.exit("bench.py --sections: the loaded library has no section census; build it with "
+                 "`python -m raygaussx_amd.build --sections` and set RGX_LIB_PATH=raygaussx_amd/librgx_sections.so")
+    out, scene, cfg = training_leg(dev, args.workload, args.steps, args.warmup, args, in_flight=args.in_flight)
+    config, n, width, height = WORKLOADS[args.workload]
+    out["valu_measured"] = valu_measured(dev)
     bw = copy_bandwidth(dev)
     out["hbm_measured"] = dict(copy_GBps=bw, what="1 GiB device-to-device copy, bytes read + written",
-                               roofline_frac_of_measured=round(dom["achieved"] / bw, 5),
+                               roofline_frac_of_measured=round(out["roofline"]["achieved"] / bw, 5),
                                step_frac_of_measured=round(out["step_roofline"]["achieved"] / bw, 5))
-    if args.fps_frames > 0 and args.workload == "c4_1M_800x800" and not args.forward_only:
+    headline = args.workload == "c4_1M_800x800" and not args.forward_only
+    if args.fps_frames > 0 and headline:
         out["fwd_fps_c3"] = inference_leg(dev, args.fps_frames, 3)
+    if args.other_steps > 0 and headline:
+        others = {}
+        for name in OTHER_WORKLOADS:
+            o, _, _ = training_leg(dev, name, args.other_steps, 2, args, in_flight=1)
+            dom = o["roofline"]
+            others[name] = dict(value=o["value"], unit="Mrays/s", ms_per_step=o["ms_per_step"], steps=o["steps"], warmup=o["warmup"],
+                                step_roofline_frac=o["step_roofline"]["frac"], roofline_mrays=o["step_roofline"]["roofline_mrays"],
+                                dominant_kernel=dom["kernel"], dominant_kernel_ms=dom["kernel_ms"], dominant_kernel_frac=dom["frac"],
+                                march_kernels={k: dict(kernel_ms=v["kernel_ms"], frac=v["frac"],
+                                                       lane_slots_per_pair_at_measured_issue_rate=v["lane_slots_per_pair_at_measured_issue_rate"])
+                                               for k, v in dom["march_kernels"].items()},
+                                hit_pairs_per_launch=dom["hit_pairs_per_launch"], kernels_ms=o["kernels_ms"], memory=o["memory"],
+                                config=o["config"])
+        out["other_workloads"] = others
     if args.cpu_rays > 0:
+        # the box grants a job 16 host threads whatever os.cpu_count() shows: the baseline uses those, and says so
         threads = min(16, os.cpu_count() or 1)
         out["cpu_baseline"] = cpu_baseline(scene, scenes.make_camera(config, 0, width=width, height=height), cfg,
                                            args.cpu_rays if n <= 1_000_000 else min(args.cpu_rays, 16384), threads,
-                                           backward=not args.forward_only)
+                                           backward=not (args.forward_only or args.workload.endswith("_fwd")))
+        out["cpu_baseline"]["host_cpus"] = os.cpu_count()
+        out["cpu_baseline"]["threads_note"] = "min(16, host cpus): 16 is this GPU box's CPU share per job"
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out), flush=True)

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define RGX_ABI_VERSION 5
+#define RGX_ABI_VERSION 6
 
 #define RGX_OK 0
 #define RGX_EINVAL -1     /* bad argument (null pointer, negative size, unsupported degree ...) */
@@ -127,12 +127,18 @@ int rgx_build_aabbs(const float *bboxes, int64_t n, void *ws, size_t ws_bytes, v
  * accel update): new boxes for the same Gaussians into a workspace that rgx_build / rgx_build_aabbs
  * built for this n.  The tree keeps its shape (sorted order, children); leaf and internal boxes and
  * the scene box are recomputed.  About a third of a build's time; queries stay exact however far the
- * Gaussians moved, the tree only culls worse the further they did. */
+ * Gaussians moved, the tree only culls worse the further they did.
+ * Precondition: `ws` holds a finished tree over exactly n boxes and `bboxes` has n rows.  The first
+ * is checked on the device, in stream order, by the refit's first kernel: when it does not hold
+ * (workspace never built, built for another n, or left unfinished) no kernel of the refit touches
+ * the tree, the workspace is left marked not built -- rgx_scene_bbox then returns RGX_EWORKSPACE --
+ * and this call still returns RGX_OK, because the host does not wait for the check. */
 int rgx_refit_aabbs(const float *bboxes, int64_t n, void *ws, size_t ws_bytes, void *stream);
 
 /* Synchronous read-back of the scene bbox held in a built workspace
  * (host out[6] = min xyz, max xyz); what bb_min.get()/bb_max.get() returned at
- * optix_utils.py:254-255.  Waits for `stream`. */
+ * optix_utils.py:254-255.  Waits for `stream`.  RGX_EWORKSPACE when the workspace holds no
+ * finished tree (never built, or a refit that was refused). */
 int rgx_scene_bbox(const void *ws, float *host_out6, void *stream);
 /* The build's permutation: order[j] = input index of the j-th Gaussian in Morton order. */
 int rgx_build_order(const void *ws, int64_t n, int32_t *order_out, void *stream);
@@ -228,8 +234,13 @@ int rgx_march_backward_noalloc(const void *ws, const RgxCamera *cam, const RgxMa
  * replaying backward did not consume its hit-list record exactly (the gradient of such a tile is
  * that of the iterations replayed so far); host_out[1]: sweeps of the tree that had to drop nodes
  * because the node stack was full (cannot happen for trees of at most 2^30 leaves; counted so that
- * it would be seen).  Both are cleared by the next rgx_march_forward / rgx_march_backward on the
- * workspace.  A workspace with room for the gradient block only keeps no counts (zeros). */
+ * it would be seen).  rgx_march_forward and rgx_march_viewer clear both at their start;
+ * rgx_march_backward clears host_out[0] at its start and adds to host_out[1], which therefore covers
+ * the forward and the backward launches since.  A backward into a workspace that no forward has used
+ * finds host_out[1] as the memory was: zero a fresh workspace's 256 bytes at offset
+ * align256(max(n, 1) * 64) first (the Python mirror allocates its workspaces zeroed).  A workspace with
+ * room for the gradient block only keeps no counts (zeros); the array of rgx_march_backward_noalloc
+ * cannot be read back. */
 int rgx_march_faults(const void *march_ws, size_t march_ws_bytes, int64_t n, uint64_t *host_out2, void *stream);
 
 /* The interactive viewer's two kernels (its GL window and interop stay with the caller).
@@ -299,6 +310,15 @@ int rgx_collect_tiles(const void *ws, const RgxCamera *cam, const float *prims, 
  * from the full sequences; *bad (device, cleared by the caller) receives the count, 0 for operands in range
  * (2^-46 <= |a|, |b| <= 2^46). */
 int rgx_check_plain_arith(const float *a, const float *b, int64_t n, uint32_t *bad, void *stream);
+
+/* Measurement hook (no counterpart in the reference): a kernel of nothing but independent fp32
+ * multiply-adds, for the rate at which this card issues VALU instructions -- the ceiling the march
+ * kernels, which are bound by instruction issue, are priced against.  Launches `waves` wavefronts
+ * (rounded up to whole workgroups of four) that each issue iters * 64 multiply-adds; *instructions
+ * (host) receives the number of VALU wave instructions the launch issues in its loops.  `sink`
+ * (device, at least one float) keeps the compiler from dropping the arithmetic; nothing is written
+ * to it for finite inputs.  The caller times the launch with events on `stream`. */
+int rgx_probe_valu_rate(int32_t waves, int32_t iters, float *sink, uint64_t *instructions, void *stream);
 
 /* ---- Morton reordering of the point cloud --------------------------------- */
 

@@ -86,6 +86,24 @@ def set_step_scale(scale):
     lib().orc_set_step_scale(C.c_float(scale))
 
 
+def set_backward_mask_form(forward_form):
+    """0: the backward's gradient loop decides ``power < k^2`` as the reference's backward does; 1: by the
+    forward's arrangement of the same arithmetic (see orc_set_backward_mask_form in rgx_oracle.c)."""
+    lib().orc_set_backward_mask_form(C.c_int(int(bool(forward_form))))
+
+
+def march_backward_in_cut(cam_struct, march, bmin, bmax, prims, ray_colors, ray_ids=None):
+    """Per ray (n, 2): samples the backward's gradient loop took as inside a Gaussian's cut-off, and samples on
+    which the reference's forward and backward arrangements of ``power`` decide differently."""
+    prims, bmin, bmax, ray_colors = _f(prims), _f(bmin), _f(bmax), _f(ray_colors)
+    ids = None if ray_ids is None else np.ascontiguousarray(ray_ids, dtype=np.int64)
+    n = cam_struct.width * cam_struct.height if ids is None else len(ids)
+    out = np.zeros((n, 2), np.int64)
+    lib().orc_march_backward_in_cut(C.byref(cam_struct), C.byref(march), _p(bmin), _p(bmax), C.c_int64(prims.shape[0]),
+                                    _p(prims), C.c_int64(0 if ids is None else len(ids)), _p(ids), _p(ray_colors), _p(out))
+    return out
+
+
 def cull_build(prims):
     """Build the oracle's optional bounding-volume tree over this primitive block (the timed CPU baseline
     uses it; results are those of the brute force).  Keep ``prims`` alive and pass the same array to the

@@ -97,6 +97,7 @@ static inline float dot3(f3 a, f3 b) { return (a.x * b.x + a.y * b.y) + a.z * b.
 static inline f3 normalize3(f3 v) { float inv = 1.0f / sqrtf(dot3(v, v)); return scl3(v, inv); }
 static inline float canon_logf(float x) { return (float)log((double)x); }
 static float g_step_scale = 1.0f; /* see orc_set_step_scale() */
+static int g_mask_form = 0;       /* see orc_set_backward_mask_form() */
 
 /* cuda_train/forward/gaussians_aabb.cu:7-17 quaternion_to_matrix (columns of R) */
 static inline void quat_to_cols(const float *q, f3 *c0, f3 *c1, f3 *c2)
@@ -898,7 +899,7 @@ static inline void acc_add(double *p, float v)
 static void march_backward_ray(const OrcCamera *cam, const OrcMarch *m, const float *bmin,
                                const float *bmax, int64_t N, const float *prims, int64_t ray,
                                const float *ray_color, const float *dloss, CandList *L,
-                               int32_t *ids, GradAcc *g, OrcStats *st)
+                               int32_t *ids, GradAcc *g, OrcStats *st, int64_t *in_cut)
 {
     const unsigned ix = (unsigned)(ray % cam->width), iy = (unsigned)(ray / cam->width);
     const f3 o = mk3(cam->eye[0], cam->eye[1], cam->eye[2]);
@@ -968,6 +969,15 @@ static void march_backward_ray(const OrcCamera *cam, const OrcMarch *m, const fl
                 const float power_cut = k * k;
                 f3 U, V, W;
                 quat_to_cols(p + 8, &U, &V, &W);
+                /* the same power by the forward's arrangement (gaussians_aabb.cu:135-164: t_mid by fmaf, the   */
+                /* dot-product form of S^-1 R^T), its recurrence carried over the slab's 32 samples: see          */
+                /* orc_set_backward_mask_form()                                                                  */
+                const f3 fx0 = apply_sinv_rt(add3(pos_rel, scl3(dir, fmaf(dt, 0.5f, tbuffer))), U, V, W, inv_s);
+                const f3 fMd = apply_sinv_rt(dir, U, V, W, inv_s);
+                const float fMd_dt_2 = (dt * dt) * dot3(fMd, fMd);
+                float fpower = dot3(fx0, fx0);
+                float finc = fMd_dt_2 + 2.0f * dot3(fx0, fMd) * dt;
+                const float finc_st = 2.0f * fMd_dt_2;
                 U = scl3(U, inv_s.x); V = scl3(V, inv_s.y); W = scl3(W, inv_s.z);
                 const f3 M1 = mk3(U.x, V.x, W.x), M2 = mk3(U.y, V.y, W.y), M3 = mk3(U.z, V.z, W.z);
                 const float gd = p[15];
@@ -987,7 +997,9 @@ static void march_backward_ray(const OrcCamera *cam, const OrcMarch *m, const fl
                         const float sigma = buffers[b][i][0];
                         const float w = expf(-sigma * dt);
                         const float e = buffers[b][i][1];
-                        if (power < power_cut) {
+                        const int in_b = power < power_cut, in_f = fpower < power_cut;
+                        if (in_cut) { in_cut[0] += in_b; in_cut[1] += in_b != in_f; }
+                        if (g_mask_form ? in_f : in_b) {
                             const float aT = Tt * (1.0f - w) * ((sigma > 0.0f) ? 1.0f / sigma : 0.0f);
                             const float wd = expf(-0.5f * power);
                             const float sw = wd * gd;
@@ -1011,6 +1023,8 @@ static void march_backward_ray(const OrcCamera *cam, const OrcMarch *m, const fl
                         Mx = add3(Mx, scl3(Md, dt));
                         power += inc;
                         inc += inc_st;
+                        fpower += finc;
+                        finc += finc_st;
                         Dt -= Tt * (1.0f - w) * e;
                         Tt *= w;
                     }
@@ -1067,7 +1081,7 @@ void orc_march_backward(const OrcCamera *cam, const OrcMarch *m, const float *bm
         for (int64_t r = 0; r < n; ++r) {
             int64_t ray = ray_ids ? ray_ids[r] : r;
             march_backward_ray(cam, m, bmin, bmax, N, prims, ray, ray_colors + 3 * ray, dloss + 3 * ray,
-                               &L, ids, &g, &st);
+                               &L, ids, &g, &st, NULL);
         }
 #pragma omp critical
         stats_add(&total, &st);
@@ -1120,6 +1134,46 @@ int orc_num_threads(void)
 /* Sensitivity probe for the tests: scales the adaptive step's coefficient (1.0f: exactly the
  * reference's arithmetic; 1 + 2^-23: as if cbrtf had rounded the other way). */
 void orc_set_step_scale(float s) { g_step_scale = s; }
+
+/* Probes of the backward's cut-off decisions (tests only).  The gradient loop of the backward
+ * (backward/gaussians_aabb.cu:375-396) decides `power < k^2` per sample from its own arrangement of
+ * the arithmetic -- the sample point by t0 = tbuffer + 0.5 dt and a 3x3 matrix product -- which is not
+ * the forward's (112-180: t_mid by fmaf, S^-1 R^T by dot products).  For a thin Gaussian one ulp of t
+ * moves the power by 1e-4 of its value, so the reference's own two passes disagree on samples that sit
+ * within that of k^2, and a sample flipped is, for a few hundred rays, 1e-3 of the whole gradient.
+ * orc_march_backward_in_cut returns per ray {samples the gradient loop took as inside a cut-off, samples on
+ * which the two arrangements disagree}; orc_set_backward_mask_form(1) makes the loop decide by the forward's
+ * arrangement (its set-up at the slab's first sample, the recurrence carried over all 32 samples), everything
+ * else as the reference has it; 0 is the reference. */
+void orc_set_backward_mask_form(int forward_form) { g_mask_form = forward_form; }
+
+void orc_march_backward_in_cut(const OrcCamera *cam, const OrcMarch *m, const float *bmin, const float *bmax,
+                               int64_t N, const float *prims, int64_t n, const int64_t *ray_ids,
+                               const float *ray_colors, int64_t *in_cut)
+{
+    GradAcc g;
+    g.ddens = (double *)calloc((size_t)N, sizeof(double));
+    g.drgb = (double *)calloc((size_t)N * 3, sizeof(double));
+    g.dpos = (double *)calloc((size_t)N * 3, sizeof(double));
+    g.dscale = (double *)calloc((size_t)N * 3, sizeof(double));
+    g.dquat = (double *)calloc((size_t)N * 4, sizeof(double));
+    if (!ray_ids) n = (int64_t)cam->width * cam->height;
+    const float zero[3] = {0.f, 0.f, 0.f};
+#pragma omp parallel
+    {
+        CandList L = {0, 0, 0};
+        int32_t *ids = (int32_t *)malloc(sizeof(int32_t) * (size_t)(m->max_prim_slice > 0 ? m->max_prim_slice : 1));
+        OrcStats st; memset(&st, 0, sizeof st);
+#pragma omp for schedule(dynamic, 16)
+        for (int64_t r = 0; r < n; ++r) {
+            int64_t ray = ray_ids ? ray_ids[r] : r;
+            in_cut[2 * r] = in_cut[2 * r + 1] = 0;
+            march_backward_ray(cam, m, bmin, bmax, N, prims, ray, ray_colors + 3 * ray, zero, &L, ids, &g, &st, in_cut + 2 * r);
+        }
+        free(ids); free(L.c);
+    }
+    free(g.ddens); free(g.drgb); free(g.dpos); free(g.dscale); free(g.dquat);
+}
 
 void orc_set_num_threads(int n)
 {

@@ -31,14 +31,14 @@ class RgxMarch(C.Structure):
 STATS_FIELDS = ("hit_pairs", "slabs", "empty_slabs", "overflow_rays", "rays_hit", "nodes_visited", "candidates",
                 "candidates_hit", "replay_lost", "grad_atomics")
 
-ABI_VERSION = 5   # RGX_ABI_VERSION of include/rgx.h
+ABI_VERSION = 6   # RGX_ABI_VERSION of include/rgx.h
 
 # every symbol include/rgx.h declares
 SYMBOLS = ("rgx_abi_version", "rgx_strerror", "rgx_last_hip_error", "rgx_aabb", "rgx_sh_forward",
            "rgx_sh_backward", "rgx_build_workspace_bytes", "rgx_build", "rgx_build_aabbs", "rgx_refit_aabbs", "rgx_scene_bbox",
            "rgx_build_order", "rgx_build_layout", "rgx_pack_prims", "rgx_march_workspace_bytes", "rgx_march_records_bytes", "rgx_march_forward", "rgx_march_forward_counts",
            "rgx_march_backward", "rgx_march_backward_noalloc", "rgx_march_faults", "rgx_first_hit", "rgx_trace_segments", "rgx_collect_tiles", "rgx_morton_workspace_bytes",
-           "rgx_morton_order", "rgx_sh_viewer", "rgx_march_viewer", "rgx_gather_rows", "rgx_knn_workspace_bytes", "rgx_dist2_knn3", "rgx_reduce_supersampling", "rgx_check_plain_arith", "rgx_timing_enable", "rgx_timing_reset", "rgx_timing_name", "rgx_timing_read")
+           "rgx_morton_order", "rgx_sh_viewer", "rgx_march_viewer", "rgx_gather_rows", "rgx_knn_workspace_bytes", "rgx_dist2_knn3", "rgx_reduce_supersampling", "rgx_check_plain_arith", "rgx_probe_valu_rate", "rgx_timing_enable", "rgx_timing_reset", "rgx_timing_name", "rgx_timing_read")
 
 _lib = None
 

@@ -11,6 +11,9 @@ bytes of register spills per lane, LDS.  The march kernels are sized for three w
 (168 registers) and twelve tiles per CU (12 800 bytes of LDS); a change that pushes spills into
 their sweep loops costs more than most optimisations gain, so look at this table after touching
 them.
+
+``python -m raygaussx_amd.build --sections`` builds ``librgx_sections.so``, a diagnostic copy whose march
+kernels count the cycles each of their sections takes (see ``bench.py --sections``).
 """
 import os
 import subprocess
@@ -81,5 +84,18 @@ def build(verbose=False, extra=(), lib=LIB, tag="", resources=False):
     return lib
 
 
+SECTIONS_LIB = os.path.join(HERE, "librgx_sections.so")
+
+
+def build_sections(**kw):
+    """The diagnostic build with the per-section cycle census of the march kernels compiled in
+    (``-DRGX_SECTION_CLOCKS``): ``librgx_sections.so`` beside the product library, which it never replaces.
+    ``RGX_LIB_PATH=raygaussx_amd/librgx_sections.so python bench.py --sections`` reads the census."""
+    return build(extra=["-DRGX_SECTION_CLOCKS"], lib=SECTIONS_LIB, tag="_sections", **kw)
+
+
 if __name__ == "__main__":
-    print(build(verbose=True, resources="--resources" in sys.argv[1:]))
+    if "--sections" in sys.argv[1:]:
+        print(build_sections(verbose=True, resources="--resources" in sys.argv[1:]))
+    else:
+        print(build(verbose=True, resources="--resources" in sys.argv[1:]))

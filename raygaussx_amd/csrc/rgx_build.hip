@@ -27,8 +27,32 @@ __global__ void k_init_header(WsHeader *h, int64_t n)
         h->n = n;
         h->root = 0;
         h->built = 0;
+        h->refit_ok = 0;
     }
 }
+
+// First kernel of a refit.  A refit walks the parent / child / order arrays the last build left in the
+// workspace, so it may only run over a finished tree of exactly n boxes: anything else (a workspace never
+// built, built for another n, or left unfinished) would send the refit kernels to indices that mean nothing.
+// The check runs on the device, in stream order after whatever build precedes it; when it fails the header is
+// left not built, `refit_ok` stays 0 and every later kernel of the refit returns at once (`gate`).
+__global__ void k_refit_begin(WsHeader *h, int64_t n)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        const bool ok = h->built == 1 && h->n == n && h->root == 0;
+        for (int a = 0; a < 3; ++a) {
+            h->bb_min_enc[a] = enc_f(INFINITY);
+            h->bb_max_enc[a] = enc_f(-INFINITY);
+            if (ok) {
+                h->bb_min[a] = INFINITY;
+                h->bb_max[a] = -INFINITY;
+            }
+        }
+        h->built = 0;
+        h->refit_ok = ok ? 1 : 0;
+    }
+}
+__device__ __forceinline__ bool gate_closed(const int32_t *gate) { return gate != nullptr && *gate == 0; }
 
 __device__ __forceinline__ float wave_min(float v)
 {
@@ -102,9 +126,10 @@ __global__ void k_decode_enc(int32_t *mn, int32_t *mx)
     }
 }
 
-__global__ void k_finish_bbox(WsHeader *h, float *bb_min, float *bb_max)
+__global__ void k_finish_bbox(WsHeader *h, float *bb_min, float *bb_max, const int32_t *gate = nullptr)
 {
     const int a = threadIdx.x;
+    if (gate_closed(gate)) return;
     if (a < 3) {
         const float mn = dec_f(h->bb_min_enc[a]), mx = dec_f(h->bb_max_enc[a]);
         h->bb_min[a] = mn;
@@ -288,10 +313,11 @@ static int radix_sort(K *k0, uint32_t *v0, K *k1, uint32_t *v1, int64_t n, int b
 // ---------------------------------------------------------------------------
 // Leaves, radix tree (Karras 2012), refit, skip links.
 __global__ __launch_bounds__(256) void k_leaves(const float *__restrict__ boxes, const uint32_t *__restrict__ order, int64_t n,
-                                                Node *__restrict__ nodes, int32_t *__restrict__ parent, int32_t *__restrict__ flags)
+                                                Node *__restrict__ nodes, int32_t *__restrict__ parent, int32_t *__restrict__ flags,
+                                                const int32_t *gate = nullptr)
 {
     const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (j >= n) return;
+    if (j >= n || gate_closed(gate)) return;
     const float *b = boxes + 6 * (int64_t)order[j];
     Node nd;
     nd.lo[0] = b[0]; nd.lo[1] = b[1]; nd.lo[2] = b[2];
@@ -368,10 +394,11 @@ __device__ __forceinline__ float ld_agent(const float *p)
 
 __global__ __launch_bounds__(256) void k_refit(int64_t n, Node *nodes, const int32_t *__restrict__ parent,
                                                const int32_t *__restrict__ right, const int32_t *__restrict__ other_end,
-                                               int32_t *flags)
+                                               int32_t *flags, const int32_t *gate = nullptr)
 {
     __shared__ float s_box[2][6][256]; // [which child][lo xyz, hi xyz][node - first leaf of the workgroup]
     __shared__ int s_arrived[256];
+    if (gate_closed(gate)) return; // the whole grid
     const int64_t b0 = (int64_t)blockIdx.x * 256, j = b0 + threadIdx.x;
     s_arrived[threadIdx.x] = 0;
     __syncthreads();
@@ -407,10 +434,18 @@ __global__ __launch_bounds__(256) void k_refit(int64_t n, Node *nodes, const int
     }
     // the rest of the way: through memory
     while (node >= 0) {
+#if defined(__gfx942__) || defined(__gfx950__)
+        // (the immediate below is the gfx9 encoding of vmcnt(0) with the other counters left alone, and the
+        // argument that the wait suffices rests on how these chips complete agent-scope atomic stores)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup"); // compiler ordering
         __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0): this thread's box stores have completed
         if (atomicAdd(&flags[node], 1) == 0) return; // the sibling subtree is not done yet
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#else
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        if (atomicAdd(&flags[node], 1) == 0) return;
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#endif
         const Node *a = &nodes[nodes[node].left];
         const Node *b = &nodes[right[node]];
         for (int c = 0; c < 3; ++c) {
@@ -422,10 +457,10 @@ __global__ __launch_bounds__(256) void k_refit(int64_t n, Node *nodes, const int
 }
 
 __global__ __launch_bounds__(256) void k_skip_links(int64_t n, Node *__restrict__ nodes, const int32_t *__restrict__ parent,
-                                                    const int32_t *__restrict__ right)
+                                                    const int32_t *__restrict__ right, const int32_t *gate = nullptr)
 {
     const int64_t id = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (id >= 2 * n - 1) return;
+    if (id >= 2 * n - 1 || gate_closed(gate)) return;
     int32_t cur = (int32_t)id, skip = -1;
     for (;;) {
         const int32_t p = parent[cur];
@@ -436,7 +471,10 @@ __global__ __launch_bounds__(256) void k_skip_links(int64_t n, Node *__restrict_
     nodes[id].skip = skip;
 }
 
-__global__ void k_mark_built(WsHeader *h) { h->built = 1; }
+__global__ void k_mark_built(WsHeader *h, const int32_t *gate = nullptr)
+{
+    if (!gate_closed(gate)) h->built = 1;
+}
 
 // ---------------------------------------------------------------------------
 static inline dim3 grid_for(int64_t n, int block) { return dim3((unsigned)((n + block - 1) / block)); }
@@ -466,8 +504,9 @@ extern "C" int rgx_build_workspace_bytes(int64_t n, size_t *bytes)
 
 // Copies caller-supplied boxes into the workspace and reduces the scene bbox.
 __global__ __launch_bounds__(256) void k_take_boxes(const float *__restrict__ in, int64_t n, float *__restrict__ boxes,
-                                                    int32_t *mn_enc, int32_t *mx_enc)
+                                                    int32_t *mn_enc, int32_t *mx_enc, const int32_t *gate = nullptr)
 {
+    if (gate_closed(gate)) return; // the whole grid
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     float b[6] = {INFINITY, INFINITY, INFINITY, -INFINITY, -INFINITY, -INFINITY};
     if (i < n)
@@ -550,6 +589,10 @@ static int build_impl(const float *pos, const float *scale, const float *quat, c
 
 // Refit: the tree's shape (children, parents, sorted order) stays as the last build into `ws` left it;
 // leaf boxes are taken from `bboxes`, internal boxes and the scene box recomputed bottom-up.
+// Precondition, checked on the device by the refit's first kernel: `ws` holds a finished tree over exactly
+// `n` boxes.  If it does not, no kernel of the refit touches the tree, the workspace is left marked not
+// built (rgx_scene_bbox then reports RGX_EWORKSPACE) and the call still returns RGX_OK: the check runs in
+// stream order and the host does not wait for it.
 extern "C" int rgx_refit_aabbs(const float *bboxes, int64_t n, void *ws, size_t ws_bytes, void *stream)
 {
     if (n < 0 || n > 0x3fffffff || !ws || (n > 0 && !bboxes)) return RGX_EINVAL;
@@ -565,15 +608,16 @@ extern "C" int rgx_refit_aabbs(const float *bboxes, int64_t n, void *ws, size_t 
     int32_t *parent = (int32_t *)(w + L.parent), *right = (int32_t *)(w + L.right), *flags = (int32_t *)(w + L.flags);
     const int32_t *other_end = (const int32_t *)(w + L.keys1); // left there by the build
     void *span = rgx_span_begin(RGX_T_BUILD, s);
-    hipLaunchKernelGGL(k_init_header, dim3(1), dim3(64), 0, s, hdr, n);
+    const int32_t *gate = &hdr->refit_ok;
+    hipLaunchKernelGGL(k_refit_begin, dim3(1), dim3(64), 0, s, hdr, n);
     if (n > 0) {
-        hipLaunchKernelGGL(k_take_boxes, grid_for(n, 256), dim3(256), 0, s, bboxes, n, boxes, hdr->bb_min_enc, hdr->bb_max_enc);
-        hipLaunchKernelGGL(k_finish_bbox, dim3(1), dim3(64), 0, s, hdr, (float *)nullptr, (float *)nullptr);
-        hipLaunchKernelGGL(k_leaves, grid_for(n, 256), dim3(256), 0, s, boxes, order, n, nodes, parent, flags);
-        if (n > 1) hipLaunchKernelGGL(k_refit, grid_for(n, 256), dim3(256), 0, s, n, nodes, parent, right, other_end, flags);
-        hipLaunchKernelGGL(k_skip_links, grid_for(2 * n - 1, 256), dim3(256), 0, s, n, nodes, parent, right);
+        hipLaunchKernelGGL(k_take_boxes, grid_for(n, 256), dim3(256), 0, s, bboxes, n, boxes, hdr->bb_min_enc, hdr->bb_max_enc, gate);
+        hipLaunchKernelGGL(k_finish_bbox, dim3(1), dim3(64), 0, s, hdr, (float *)nullptr, (float *)nullptr, gate);
+        hipLaunchKernelGGL(k_leaves, grid_for(n, 256), dim3(256), 0, s, boxes, order, n, nodes, parent, flags, gate);
+        if (n > 1) hipLaunchKernelGGL(k_refit, grid_for(n, 256), dim3(256), 0, s, n, nodes, parent, right, other_end, flags, gate);
+        hipLaunchKernelGGL(k_skip_links, grid_for(2 * n - 1, 256), dim3(256), 0, s, n, nodes, parent, right, gate);
     }
-    hipLaunchKernelGGL(k_mark_built, dim3(1), dim3(1), 0, s, hdr);
+    hipLaunchKernelGGL(k_mark_built, dim3(1), dim3(1), 0, s, hdr, gate);
     rgx_span_end(span, s);
     RGX_LAUNCH_CHECK();
     return RGX_OK;
@@ -598,9 +642,14 @@ extern "C" int rgx_scene_bbox(const void *ws, float *host_out6, void *stream)
 {
     const DeviceScope on_device(ws);
     if (!ws || !host_out6) return RGX_EINVAL;
-    const WsHeader *hdr = (const WsHeader *)ws;
-    RGX_HIP(hipMemcpyAsync(host_out6, hdr->bb_min, 6 * sizeof(float), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    WsHeader h;
+    RGX_HIP(hipMemcpyAsync(&h, ws, sizeof h, hipMemcpyDeviceToHost, (hipStream_t)stream));
     RGX_HIP(hipStreamSynchronize((hipStream_t)stream));
+    if (h.built != 1) return RGX_EWORKSPACE; // never built, or a refit that found no tree of its size to refit
+    for (int a = 0; a < 3; ++a) {
+        host_out6[a] = h.bb_min[a];
+        host_out6[3 + a] = h.bb_max[a];
+    }
     return RGX_OK;
 }
 

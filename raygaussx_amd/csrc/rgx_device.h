@@ -115,6 +115,8 @@ struct __align__(16) WsHeader {
     int64_t n;
     int32_t root;
     int32_t built;
+    int32_t refit_ok; // set by a refit's first kernel: the workspace held a finished tree over the same number of boxes
+    int32_t pad_[3];
 };
 
 struct WsLayout {

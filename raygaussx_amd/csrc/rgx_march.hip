@@ -82,6 +82,56 @@ struct MarchParams {
     uint32_t *ray_counts;   // counting forward only: per ray, slabs blended and the sum of their hit-list lengths; or null
 };
 
+// Section census (diagnostic builds only: -DRGX_SECTION_CLOCKS, `python -m raygaussx_amd.build --sections`;
+// the product library has none of it).  Every wave of a kernel launched without a statistics block keeps
+// one running time stamp; RGX_SEC(cn, k) adds the cycles since the previous stamp to section k, so the
+// sections of a wave add up to its lifetime.  At its end a wave adds its sections to a device table that
+// rgx_debug_section_cycles() reads back.
+#ifdef RGX_SECTION_CLOCKS
+#define RGX_NSEC 12
+enum { RGX_SEC_SWEEP = 0, RGX_SEC_FILTER = 1, RGX_SEC_SHADE = 2, RGX_SEC_LISTS = 3, RGX_SEC_BLEND = 4, RGX_SEC_SUMS = 5,
+       RGX_SEC_SETUP = 6, RGX_SEC_TOP = 7, RGX_SEC_END = 8, RGX_SEC_EPILOGUE = 9, RGX_SEC_WALK = 10, RGX_SEC_FLUSH = 11 };
+enum { RGX_SECK_FWD_RECORD = 0, RGX_SECK_FWD_PLAIN = 1, RGX_SECK_BWD_SUMS = 2, RGX_SECK_BWD_LISTS = 3, RGX_SECK_BWD_TREE = 4, RGX_NSECK = 5 };
+#define RGX_SEC_ROWS 65536 // workgroups per launch the table has rows for (a 1920x1080 launch has 33 024)
+// [forward / backward][workgroup][section]; word RGX_NSEC of a row counts the waves that used it, the next word names their kernel.
+// The sums live in memory, not in registers: the march kernels have no registers to spare, and a census that made them
+// spill would time another kernel.
+__device__ unsigned g_section_cycles[2][RGX_SEC_ROWS][16];
+struct SectionClock {
+    unsigned last = 0;
+    unsigned *row = nullptr;
+    __device__ __forceinline__ void start(int pass)
+    {
+        row = blockIdx.x < RGX_SEC_ROWS ? g_section_cycles[pass][blockIdx.x] : nullptr;
+        last = (unsigned)__builtin_readcyclecounter();
+    }
+    __device__ __forceinline__ void to(int k)
+    {
+        const unsigned now = (unsigned)__builtin_readcyclecounter();
+        if (threadIdx.x == 0 && row) atomicAdd(row + k, now - last);
+        last = now;
+    }
+    __device__ __forceinline__ void flush(int kernel)
+    {
+        if (threadIdx.x != 0 || !row) return;
+        atomicAdd(row + RGX_NSEC, 1u);
+        row[RGX_NSEC + 1] = (unsigned)kernel;
+    }
+};
+struct NoSectionClock {
+    __device__ __forceinline__ void start(int) {}
+    __device__ __forceinline__ void to(int) {}
+    __device__ __forceinline__ void flush(int) {}
+};
+#define RGX_SEC(cn, k) (cn).clock.to(k)
+#define RGX_SEC_START(cn, pass) (cn).clock.start(pass)
+#define RGX_SEC_FLUSH(cn, kernel) (cn).clock.flush(kernel)
+#else
+#define RGX_SEC(cn, k) ((void)0)
+#define RGX_SEC_START(cn, pass) ((void)0)
+#define RGX_SEC_FLUSH(cn, kernel) ((void)0)
+#endif
+
 // Launch statistics (RgxStats).  Kernels launched without a statistics block carry none of it:
 // the counters live in registers for the whole march, and the march has none to spare.
 struct Counters {
@@ -90,6 +140,9 @@ struct Counters {
     unsigned cands = 0, cands_hit = 0; // per wave (lane 0 counts)
     unsigned replay_lost = 0;          // per wave: the backward's replay did not consume its record exactly
     unsigned grad_atomics = 0;         // fp32 atomic adds to the gradient block in memory
+#ifdef RGX_SECTION_CLOCKS
+    NoSectionClock clock;              // the census is taken on the kernels without counters
+#endif
 };
 struct NoCount { // accepts what the kernels do to a counter, keeps nothing
     template <typename T>
@@ -101,6 +154,9 @@ struct NoCount { // accepts what the kernels do to a counter, keeps nothing
 };
 struct NoCounters {
     NoCount hit_pairs, slabs, empty, overflow, rays_hit, nodes, cands, cands_hit, replay_lost, grad_atomics;
+#ifdef RGX_SECTION_CLOCKS
+    SectionClock clock;
+#endif
 };
 template <bool STATS>
 using CountersFor = typename std::conditional<STATS, Counters, NoCounters>::type;
@@ -385,7 +441,7 @@ __device__ __forceinline__ void frustum_cut(const MarchParams &P, Frustum &F, fl
         int32_t left = 0, right = 0;
         if ((uint32_t)node < n_nodes) {
             const float4 a = nodes4[2 * node], b = nodes4[2 * node + 1];
-            right = P.right[min(node, (int32_t)P.n - 2)]; // with the box, not after the test
+            right = P.right[max(0, min(node, (int32_t)P.n - 2))]; // with the box, not after the test (n = 1: no internal node, word 0 of the padded array)
             if (frustum_overlaps(F, a, b)) {
                 left = __float_as_int(a.w);
                 inner = left >= 0;
@@ -510,7 +566,7 @@ __device__ int sweep_next(const MarchParams &P, Sweep &S, const Frustum &F, int3
         if ((uint32_t)node < n_nodes) {
             const float4 a = nodes4[2 * node], b = nodes4[2 * node + 1];
             // the right child is fetched along with the box, not after the test: one memory round trip per step, not two
-            right = P.right[min(node, (int32_t)P.n - 2)];
+            right = P.right[max(0, min(node, (int32_t)P.n - 2))];
             if (frustum_overlaps(F, a, b)) {
                 left = __float_as_int(a.w);
                 leaf_hit = left < 0;
@@ -1084,11 +1140,13 @@ struct Recorder {
     {
         slot = -1;
         if (!on()) return;
-        if (blends && sums) {
+        if (blends && P.sum_next) {
+            // every blending iteration asks, also those of a tile that has gone without once: the counter then
+            // ends at the launch's whole demand, which is what the next record of this view's shape is sized from
             uint32_t s = 0;
             if (threadIdx.x == 0) s = atomicAdd(P.sum_next, 1u);
             s = (uint32_t)__builtin_amdgcn_readfirstlane((int)s);
-            if (s < (uint32_t)P.sum_slots) slot = (int)s;
+            if (sums && s < (uint32_t)P.sum_slots) slot = (int)s;
             else sums = false;
         }
         uint32_t *it = reg + off;
@@ -1178,8 +1236,10 @@ struct ReplayLds {
     uint8_t *rowlist;  // [4][RGX_CCAP]: the slot lists of the LISTS item whose gradient pass is running
 };
 
-__device__ __forceinline__ void replay_flush(const MarchParams &P, const ReplayLds &RL)
+template <typename Cn>
+__device__ __forceinline__ void replay_flush(const MarchParams &P, const ReplayLds &RL, Cn &cn)
 {
+    RGX_SEC(cn, RGX_SEC_WALK);
     __syncthreads();
     for (int slot = threadIdx.x; slot < RGX_CCAP; slot += 64) {
         const uint32_t word = RL.pid[slot];
@@ -1199,13 +1259,15 @@ __device__ __forceinline__ void replay_flush(const MarchParams &P, const ReplayL
         }
     }
     __syncthreads();
+    RGX_SEC(cn, RGX_SEC_FLUSH);
 }
 
 // Makes the WINDOW item at `at` the current window (sums of the previous one go to memory first).
-__device__ __forceinline__ void replay_window(const MarchParams &P, const ReplayLds &RL, const uint32_t *reg, int at, int &win_at)
+template <typename Cn>
+__device__ __forceinline__ void replay_window(const MarchParams &P, const ReplayLds &RL, const uint32_t *reg, int at, int &win_at, Cn &cn)
 {
     if (at == win_at) return;
-    replay_flush(P, RL);
+    replay_flush(P, RL, cn);
     const int C = (int)(uni_u32(reg[at]) & 0xffffu);
     for (int i = threadIdx.x; i < C && i < RGX_CCAP; i += 64) {
         const uint32_t pid = min(reg[at + 4 + i], (uint32_t)(P.n - 1));
@@ -1374,6 +1436,7 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
             else lo = wave_min_all(run && tmid < thi ? fmaxf(tlo, tmid) : INFINITY), hi = wave_max_all(run ? thi : -INFINITY);
             if (!(lo <= hi)) break; // no ray reaches into the second half
         }
+        RGX_SEC(cn, RGX_SEC_TOP);
         Sweep S = {0, 0};
         if (!reuse) {
             float wend = hi;
@@ -1417,7 +1480,9 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                 first = false;
                 more = !done;
             }
+            RGX_SEC(cn, RGX_SEC_SWEEP);
             if (phase == 0 && !reuse) rec.write_window(L, C);
+            RGX_SEC(cn, RGX_SEC_LISTS);
             if (phase == 0 || !Wn.resident || split) {
                 // phase 0 asks the lane's real question; a phase-1 re-filter only recounts the slab hits
                 const float cover = split ? hi : (Wn.resident ? Wn.hi : t1); // this iteration's tables cover [t0, cover]
@@ -1448,11 +1513,13 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                     q0 = cnt;
                     qov = cut;
                 }
+                RGX_SEC(cn, RGX_SEC_FILTER);
                 if (phase == 0) {
                     found = best;
                     searched_to = fmaxf(Q.slo, Q.shi); // a split phase may end before a searching ray's start
                     rec.write_lists(L, len, !more);
                 }
+                RGX_SEC(cn, RGX_SEC_LISTS);
             }
             if constexpr (WALK == WALK_FORWARD) {
                 static_assert(std::is_same<BodyA, BodyB>::value, "the forward shades both halves with one body");
@@ -1468,9 +1535,11 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
                 if (phase == 0) shade_rows(P, L, len, run, body_a);
                 else shade_rows(P, L, len, run, body_b);
             }
+            RGX_SEC(cn, RGX_SEC_SHADE);
         }
         if (phase == 0) {
             rec.write_trailer(P, any_search, split ? hi : (Wn.resident ? Wn.hi : t1), found, __any(need && p0 > 0));
+            RGX_SEC(cn, RGX_SEC_LISTS);
             run = mid(split);
             if (!__any(run)) break;
         }
@@ -1499,9 +1568,9 @@ struct Replayer {
     // The backward's iteration driven by the record instead of the tree: body_a per ray over the
     // recorded lists, once per half of the samples; mid(); body_b over the lists row by row.
     // SUMS: body_a(slot) reads the iteration's sample sums instead of walking the lists for them
-    template <bool SUMS, typename BodyA, typename Mid, typename BodyB>
+    template <bool SUMS, typename Cn, typename BodyA, typename Mid, typename BodyB>
     __device__ __forceinline__ bool slab(const MarchParams &P, const RayState &R, bool need, int &p0, float &found,
-                                         float &searched_to, BodyA body_a, Mid mid, BodyB body_b)
+                                         float &searched_to, Cn &cn, BodyA body_a, Mid mid, BodyB body_b)
     {
         const int start = at;
         int end = at; // the iteration's TRAIL item
@@ -1528,7 +1597,7 @@ struct Replayer {
             for (int a = start; a < end;) {
                 const uint32_t head = uni_u32(reg[a]);
                 if ((head & 0xff000000u) == RGX_REC_WINDOW) {
-                    replay_window(P, RL, reg, a, win_at); // later iterations of the window carry no WINDOW item
+                    replay_window(P, RL, reg, a, win_at, cn); // later iterations of the window carry no WINDOW item
                     a += 4 + (((int)(head & 0xffffu) + 3) & ~3);
                 } else {
                     a += replay_lists<true, WALK_NONE>(P, RL, reg + a, need, p0, none);
@@ -1547,7 +1616,7 @@ struct Replayer {
             for (int a = start; a < end;) {
                 const uint32_t head = uni_u32(reg[a]);
                 if ((head & 0xff000000u) == RGX_REC_WINDOW) {
-                    replay_window(P, RL, reg, a, win_at);
+                    replay_window(P, RL, reg, a, win_at, cn);
                     a += 4 + (((int)(head & 0xffffu) + 3) & ~3);
                 } else {
                     replay_lists<true, 0>(P, RL, reg + a, need, p0, body_a);
@@ -1564,7 +1633,7 @@ struct Replayer {
             for (int b = start; b < end;) {
                 const uint32_t head = uni_u32(reg[b]);
                 if ((head & 0xff000000u) == RGX_REC_WINDOW) {
-                    replay_window(P, RL, reg, b, win_at);
+                    replay_window(P, RL, reg, b, win_at, cn);
                     b += 4 + (((int)(head & 0xffffu) + 3) & ~3);
                 } else {
                     b += replay_lists<false, WALK_ROWS_ALL>(P, RL, reg + b, run, dummy, body_b);
@@ -1617,6 +1686,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
     CountersFor<STATS> cn;
+    RGX_SEC_START(cn, 0);
     Frustum F;
     frustum_planes(P.cam, px0, py0, F);
     RayState R;
@@ -1625,6 +1695,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
     const f3 dir = R.dir;
     float Cr = 0.f, Cg = 0.f, Cb = 0.f, depth = 0.f;
     Window Wn = {0.f, 0, false, 4, false, false};
+    RGX_SEC(cn, RGX_SEC_SETUP);
 
     while (__any(R.active)) {
         float tlo, thi;
@@ -1703,7 +1774,9 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
             auto second_half = [&](bool split) { // split: the hits of the second half are not known yet
                 const bool has = need && (p0 > 0 || split);
                 if (has) blend(false);
+                RGX_SEC(cn, RGX_SEC_BLEND);
                 keep_sums(0);
+                RGX_SEC(cn, RGX_SEC_SUMS);
                 // samples 16..31, only for rays still above the transmittance floor (gaussians_aabb.cu:190)
 #pragma unroll
                 for (int i = 0; i < RGX_CHUNK_SIZE; ++i) sg[i] = cr[i] = cg[i] = cb[i] = 0.f;
@@ -1712,8 +1785,11 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
             };
             const bool run2 = slab_tables<WALK_FORWARD>(P, L, F, Wn, R, need, tlo, thi, p0, ov, found, searched_to, cn, rec, accumulate,
                                           second_half, accumulate);
+            RGX_SEC(cn, RGX_SEC_TOP); // (what slab_tables did after its last section: nothing to speak of)
             if (run2) blend(true);
+            RGX_SEC(cn, RGX_SEC_BLEND);
             keep_sums(RGX_CHUNK_SIZE);
+            RGX_SEC(cn, RGX_SEC_SUMS);
             if (need && p0 > 0) {
                 cn.slabs++;
                 cn.hit_pairs += p0;
@@ -1721,6 +1797,7 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
             if (ov) cn.overflow++;
         }
         slab_end(R, need, p0, found, searched_to, cn);
+        RGX_SEC(cn, RGX_SEC_END);
     }
     if (valid) {
         const int64_t ray = (int64_t)py * P.cam.width + px;
@@ -1743,6 +1820,8 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
     }
     rec.finish(P);
     flush_stats(P.stats, cn);
+    RGX_SEC(cn, RGX_SEC_EPILOGUE);
+    RGX_SEC_FLUSH(cn, RECORD ? RGX_SECK_FWD_RECORD : RGX_SECK_FWD_PLAIN);
 }
 
 // sum over the 16 lanes of each row, left in every lane of the row.  (Every lane of these four
@@ -1811,6 +1890,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
     lane_pixel(px0, py0, px, py);
     const bool valid = px < P.cam.width && py < P.cam.height;
     CountersFor<STATS> cn;
+    RGX_SEC_START(cn, 1);
     RayState R;
     // a replay follows the forward's iteration sequence, so it takes the forward's conventions
     // (reciprocal multiply in the bbox test, clipped slab bounds)
@@ -1831,6 +1911,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
         int p0 = 0;
         bool ov = false;
         float found = -1.0f, searched_to = 0.f;
+        RGX_SEC(cn, RGX_SEC_TOP);
         if (__any(need || (R.active && R.searching))) {
             const float dt = R.dt, tbuffer = R.tbuffer;
             // (1) s_k and g.c~_k  -> PA, PB
@@ -1861,6 +1942,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
             };
             // (1') the same from the forward's sample sums: PA = sum rho w, PB = g . sum rgb rho w
             auto load_sums = [&](const float4 *slot) {
+                RGX_SEC(cn, RGX_SEC_WALK);
                 const float *dens = (const float *)slot + lane;
                 const float *col = (const float *)slot + RGX_BUFFER_SIZE * 64 + lane * 3;
 #pragma unroll
@@ -1876,12 +1958,14 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                 for (int i = 0; i < RGX_BUFFER_SIZE; ++i)
                     PB[i] = fmaf(g.x, h16(__builtin_nontemporal_load(col + i * 192)),
                                  fmaf(g.y, h16(__builtin_nontemporal_load(col + i * 192 + 1)), g.z * h16(__builtin_nontemporal_load(col + i * 192 + 2))));
+                RGX_SEC(cn, RGX_SEC_SUMS);
             };
             // (2) prefix: PA <- a_k, PB <- (T_k e_k - D_k) dt - a_k e_k   (so X_k = PB + PA * g.c_i);
             // it always covers all 32 samples (330-352)
             float T_after = R.T, D_after = D;
             bool use_second = true; // transmittance at the chunk boundary gates the second chunk (398)
             auto prefix = [&](bool) {
+                RGX_SEC(cn, RGX_SEC_WALK);
                 const bool has = need && p0 > 0;
                 if (has) {
                     float T_mid = R.T;
@@ -1900,11 +1984,13 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                     }
                     use_second = T_mid > P.m.t_eps;
                 }
+                RGX_SEC(cn, RGX_SEC_BLEND);
                 return has;
             };
             // (3) per table entry: moments per lane, row sum, one set of atomics per row
             auto gradients = [&](const auto &e, bool hit, bool live, auto which) {
                 constexpr int GROUP = decltype(which)::group; // lanes that share this trip's entry
+                RGX_SEC(cn, RGX_SEC_WALK);
                 float out[RGX_NSUM];
 #pragma unroll
                 for (int c = 0; c < RGX_NSUM; ++c) out[c] = 0.f;
@@ -1977,6 +2063,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                         cn.grad_atomics += 14;
                     }
                 }
+                RGX_SEC(cn, RGX_SEC_SHADE);
             };
             bool has;
             if constexpr (SUMS) has = drive(need, tlo, thi, p0, ov, found, searched_to, load_sums, prefix, gradients);
@@ -1989,17 +2076,20 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
             }
             if (ov) cn.overflow++;
         }
+        RGX_SEC(cn, RGX_SEC_WALK);
         slab_end(R, need, p0, found, searched_to, cn);
+        RGX_SEC(cn, RGX_SEC_END);
     };
 
+    RGX_SEC(cn, RGX_SEC_SETUP);
     if constexpr (REPLAY) {
         Replayer rp = {reg, min((int)uni_u32(reg[1]), P.rec_tile_words), 4, -1, false, RL};
         while (__any(R.active) && !rp.lost) {
             iteration([&](bool need, float, float, int &p0, bool &, float &found, float &searched_to, auto a, auto mid, auto b) {
-                return rp.template slab<SUMS>(P, R, need, p0, found, searched_to, a, mid, b);
+                return rp.template slab<SUMS>(P, R, need, p0, found, searched_to, cn, a, mid, b);
             });
         }
-        replay_flush(P, RL);
+        replay_flush(P, RL, cn);
         if ((rp.lost || rp.at != rp.used) && lane == 0) {
             cn.replay_lost = 1;
             if (P.faults) atomicAdd(&P.faults[0], 1u); // counted with or without a statistics block
@@ -2017,6 +2107,8 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
         }
     }
     flush_stats(P.stats, cn);
+    RGX_SEC(cn, RGX_SEC_EPILOGUE);
+    RGX_SEC_FLUSH(cn, REPLAY ? (SUMS ? RGX_SECK_BWD_SUMS : RGX_SECK_BWD_LISTS) : RGX_SECK_BWD_TREE);
 }
 
 // Launch order of the replaying backward.  A tile is one wavefront's work from start to end, so a
@@ -2536,6 +2628,7 @@ static int march_backward_launch(const void *ws, const RgxCamera *cam, const Rgx
     P.dloss = dloss;
     hipStream_t s = (hipStream_t)stream;
     hipLaunchKernelGGL(k_zero4, grid_for(4 * n, 256), dim3(256), 0, s, (float4 *)P.gbuf, 4 * n);
+    if (P.faults) hipLaunchKernelGGL(k_zero_u32, dim3(1), dim3(256), 0, s, P.faults, 1); // this launch's replays that lost their record
     void *span = timed ? rgx_span_begin(RGX_T_MARCH_BWD, s) : nullptr;
     if (P.records) {
         // tiles with a complete record replay it; the few whose record overflowed are recomputed
@@ -2642,6 +2735,32 @@ extern "C" int rgx_collect_tiles(const void *ws, const RgxCamera *cam, const flo
     return RGX_OK;
 }
 
+#ifdef RGX_SECTION_CLOCKS
+// Diagnostic builds only: the section census since the last reset, summed over workgroups and launches per kernel:
+// host_out[kernel][section] cycles and host_out[kernel][RGX_NSEC] waves (RGX_NSECK x (RGX_NSEC + 1) words).  Waits for the device.
+extern "C" int rgx_debug_section_cycles(unsigned long long *host_out, int reset)
+{
+    RGX_HIP(hipDeviceSynchronize());
+    if (host_out) {
+        static unsigned host[2][RGX_SEC_ROWS][16];
+        RGX_HIP(hipMemcpyFromSymbol(host, HIP_SYMBOL(g_section_cycles), sizeof(host)));
+        for (int i = 0; i < RGX_NSECK * (RGX_NSEC + 1); ++i) host_out[i] = 0;
+        for (int pass = 0; pass < 2; ++pass)
+            for (int r = 0; r < RGX_SEC_ROWS; ++r) {
+                const unsigned *row = host[pass][r];
+                if (!row[RGX_NSEC] || row[RGX_NSEC + 1] >= RGX_NSECK) continue;
+                for (int k = 0; k <= RGX_NSEC; ++k) host_out[row[RGX_NSEC + 1] * (RGX_NSEC + 1) + k] += row[k];
+            }
+    }
+    if (reset) {
+        void *p = nullptr;
+        RGX_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_section_cycles)));
+        RGX_HIP(hipMemset(p, 0, sizeof(unsigned) * 2 * RGX_SEC_ROWS * 16));
+    }
+    return RGX_OK;
+}
+#endif
+
 // Test hook: counts the pairs for which the plain division or the plain square root differs in any
 // bit from `/` or sqrtf() (expected: none, for operands inside the ranges plain_roots() grants).
 __global__ __launch_bounds__(256) void k_check_plain_arith(const float *__restrict__ a, const float *__restrict__ b, int64_t n,
@@ -2662,6 +2781,37 @@ extern "C" int rgx_check_plain_arith(const float *a, const float *b, int64_t n, 
     const DeviceScope on_device(a);
     if (n < 0 || (n > 0 && (!a || !b)) || !bad) return RGX_EINVAL;
     if (n > 0) hipLaunchKernelGGL(k_check_plain_arith, grid_for(n, 256), dim3(256), 0, (hipStream_t)stream, a, b, n, bad);
+    RGX_LAUNCH_CHECK();
+    return RGX_OK;
+}
+
+// Measurement hook: independent fp32 multiply-adds and nothing else (16 chains per lane, so that no
+// instruction waits for the one before), for the VALU issue rate of the card.
+__global__ __launch_bounds__(256) void k_probe_valu(int iters, float seed, float *sink)
+{
+    float a[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) a[i] = seed + (float)(threadIdx.x + i);
+    const float m = 1.0f - seed * 1e-9f, c = seed * 1e-9f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) a[i] = fmaf(a[i], m, c);
+    }
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) t += a[i];
+    if (t == -1.2345f) *sink = t; // never for finite seeds: the sums stay positive
+}
+
+extern "C" int rgx_probe_valu_rate(int32_t waves, int32_t iters, float *sink, uint64_t *instructions, void *stream)
+{
+    if (waves <= 0 || iters <= 0 || !sink || !instructions) return RGX_EINVAL;
+    const DeviceScope on_device(sink);
+    const unsigned groups = (unsigned)((waves + 3) / 4);
+    hipLaunchKernelGGL(k_probe_valu, dim3(groups), dim3(256), 0, (hipStream_t)stream, (int)iters, 1.0f, sink);
+    *instructions = (uint64_t)groups * 4u * (uint64_t)iters * 64u;
     RGX_LAUNCH_CHECK();
     return RGX_OK;
 }

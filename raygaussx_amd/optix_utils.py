@@ -29,7 +29,7 @@ def _workspace(key, nbytes, device):
     slot = (key, str(device), torch.cuda.current_stream(device).cuda_stream)
     t = _scratch.pop(slot, None)
     if t is None or t.numel() < nbytes:
-        t = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        t = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)   # zeroed: the fault counters start at 0
     _scratch[slot] = t          # re-inserted: dicts keep insertion order, so this is now the newest
     mine = [k for k in _scratch if k[0] == key and k[1] == str(device)]
     for k in mine[:-_SCRATCH_STREAMS]:
@@ -53,8 +53,10 @@ class AccelerationStructure:
     def __init__(self, n, device):
         self.n = int(n)
         self.device = device
+        self.built = False      # a build has been queued into ``ws``: only then is there a tree to refit
         nbytes = L.size_query(L.lib().rgx_build_workspace_bytes, C.c_int64(self.n))
         self.ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        self.ws[:256].zero_()   # the header: "not built" until a build has finished
 
     @property
     def handle(self):
@@ -64,16 +66,28 @@ class AccelerationStructure:
         L.check(L.lib().rgx_build(L.ptr(positions), L.ptr(scales), L.ptr(quaternions), L.ptr(densities),
                                   C.c_int64(self.n), C.c_float(SIGMA_THRESHOLD), L.ptr(self.ws),
                                   C.c_size_t(self.ws.numel()), L.stream(self.device)))
+        self.built = True
         return self
 
     def build_from_boxes(self, bboxes):
+        bboxes = L.f32(bboxes)
+        if tuple(bboxes.shape) != (self.n, 6):
+            raise L.RgxError(f"librgx: {self.n} boxes expected as an ({self.n}, 6) tensor, got {tuple(bboxes.shape)}")
         L.check(L.lib().rgx_build_aabbs(L.ptr(bboxes), C.c_int64(self.n), L.ptr(self.ws),
                                         C.c_size_t(self.ws.numel()), L.stream(self.device)))
+        self.built = True
         return self
 
     def update(self, bboxes):
-        """New boxes for the same Gaussians: refit (the tree keeps its shape), as OptiX's accel update does."""
+        """New boxes for the same Gaussians: refit (the tree keeps its shape), as OptiX's accel update does.
+        Only a structure that was built can be updated, and only with one box per Gaussian of that build: the
+        refit walks the tree the build left in the workspace."""
+        if not self.built:
+            raise L.RgxError("librgx: update of an acceleration structure that was never built")
         bboxes = L.f32(bboxes)
+        if tuple(bboxes.shape) != (self.n, 6) or bboxes.device != self.ws.device:
+            raise L.RgxError(f"librgx: update needs an ({self.n}, 6) tensor of boxes on {self.ws.device}, got "
+                             f"{tuple(bboxes.shape)} on {bboxes.device}")
         L.check(L.lib().rgx_refit_aabbs(L.ptr(bboxes), C.c_int64(self.n), L.ptr(self.ws), C.c_size_t(self.ws.numel()),
                                         L.stream(self.device)))
         return self
@@ -198,7 +212,12 @@ def _march_ws(n, n_rays, max_prim_slice, device):
 # Record size per 8x8 pixel tile, 32-bit words: 16384 for the hit lists (64 KiB) and on average 64
 # slots of 8192 words for the per-sample density and colour sums of a slab iteration (the slots are
 # one pool shared by all tiles).  2.06 MiB per tile: 21 GB at 800x800.  16384 keeps the hit lists only.
+# This is the most a record holds; what a launch is given is sized from use (new_records).
 REC_TILE_WORDS = 16384 + 64 * 8192
+# The first view of a scene size and image shape on a stream, of which nothing is known yet, gets a pool of
+# this many slots per tile: its forward counts the slots it would have used, tiles that find the pool empty
+# are replayed from their hit lists (slower, same gradients), and the second view's pool is sized from the count.
+REC_FIRST_SLOTS = 12
 
 
 REC_LIST_WORDS = 16384        # the hit lists' share of a tile's record
@@ -224,14 +243,19 @@ def fit_tile_words(cam, tile_words, budget_bytes):
     return lists + slots * REC_SLOT_WORDS if (tile_words > lists and slots >= 1) else lists
 
 
-# What the forward launches of one image size actually took from the sample-sum pool, so that the next
-# record of that size is allocated for the need instead of for 64 slots per tile:
-# (device, width, height) -> {"pinned": host int32[1], "event", "pending", "need": slots of the last views,
-#                             "slots": the pool size in use, "allocated": bytes of the last record}
+# What the forward launches of one scene size and image shape on one stream asked of the sample-sum pool
+# (the launch's whole demand: every blending slab iteration asks, served or not), so that the next record
+# is allocated for the need:
+# (device, stream, Gaussians, width, height) -> {"pinned": host int32[1], "event", "pending", "need": slots the
+#                             last views asked for, "slots": the pool size in use, "allocated": bytes of the last record}
 _rec_usage = {}
 REC_POOL_MARGIN = 1.05        # pool = this times the largest need of the last views ...
-REC_POOL_STEP = 1 << 15       # ... rounded up to a multiple of this many slots (1 GiB), so that the size stays put
+REC_POOL_STEP = 1 << 12       # ... rounded up to a multiple of this many slots (128 MiB), so that the size stays put
 REC_POOL_HISTORY = 8
+
+
+def _usage_key(cam, device, n):
+    return (str(device), torch.cuda.current_stream(device).cuda_stream, int(n), cam.width, cam.height)
 
 
 def _pool_geometry(cam):
@@ -239,30 +263,38 @@ def _pool_geometry(cam):
     return ntiles, ntiles * REC_LIST_WORDS * 4        # tiles, bytes of the hit-list regions (the pool header follows)
 
 
-def new_records(cam, device, tile_words=REC_TILE_WORDS, budget_bytes=None):
+def new_records(cam, device, tile_words=REC_TILE_WORDS, budget_bytes=None, n=0):
     """Buffer for the record of one forward launch (see rgx_march_records_bytes), or None when no
     record fits the budget or the allocator.  The budget defaults to REC_MEMORY_SHARE of the device's
     memory and at most 80 % of what is free now.  With the default ``tile_words`` the pool of sample
-    sums is sized from what the last forward launches of this image size took from it
-    (``note_record_use``) instead of the 64 slots per tile of a first call: tiles that find the pool
-    empty are replayed from their hit lists alone, so a guess that is too small costs time, not
-    correctness, and the next record grows."""
+    sums is sized from what the last forward launches of this scene size (``n`` Gaussians) and image
+    shape on this stream asked for (``note_record_use``); the first such view, of which nothing is
+    known, gets REC_FIRST_SLOTS slots per tile.  Tiles that find the pool empty are replayed from
+    their hit lists alone, so a pool that is too small costs time, not correctness, and the forward's
+    count of what it would have used sizes the next one."""
     if budget_bytes is None:
         free, total = torch.cuda.mem_get_info(device)
         budget_bytes = int(min(REC_MEMORY_SHARE * total, 0.8 * free))
-    use = _rec_usage.get((str(device), cam.width, cam.height))
-    if tile_words == REC_TILE_WORDS and use is not None and use["need"]:
+    if tile_words == REC_TILE_WORDS:
+        key = _usage_key(cam, device, n)
+        use = _rec_usage.get(key)
+        if use is None:
+            if len(_rec_usage) >= 64:
+                del _rec_usage[next(iter(_rec_usage))]
+            use = _rec_usage[key] = dict(pinned=torch.zeros(1, dtype=torch.int32).pin_memory(), event=torch.cuda.Event(),
+                                         pending=False, need=[], slots=0, allocated=0)
         _read_record_use(use)
         ntiles, head = _pool_geometry(cam)
-        have = use.get("slots", 0)
-        need = max(use["need"])
-        # a launch that ran the pool dry stops counting tile by tile, so its count is a lower bound: grow faster
-        want = int(need * (1.5 if have and need >= have else REC_POOL_MARGIN)) + 1
-        if want > have or want * 1.5 < have:      # grow when short; shrink only when far too large
-            have = (want + REC_POOL_STEP - 1) // REC_POOL_STEP * REC_POOL_STEP
-        have = min(have, 64 * ntiles)
+        have = use["slots"]
+        if use["need"]:
+            want = int(max(use["need"]) * REC_POOL_MARGIN) + 1
+            if want > have or want * 1.5 < have:      # grow when short; shrink only when far too large
+                have = (want + REC_POOL_STEP - 1) // REC_POOL_STEP * REC_POOL_STEP
+        elif not have:
+            have = REC_FIRST_SLOTS * ntiles
+        have = max(min(have, 64 * ntiles), ntiles)     # (the library wants at least one slot per tile to keep sums at all)
         nbytes = head + 256 + have * REC_SLOT_WORDS * 4
-        if have > ntiles and nbytes <= budget_bytes:
+        if nbytes <= budget_bytes:
             try:
                 rec = torch.empty(nbytes, dtype=torch.uint8, device=device)
                 use["slots"] = have
@@ -284,20 +316,15 @@ def _read_record_use(use):
         use["need"] = (use["need"] + [int(use["pinned"][0])])[-REC_POOL_HISTORY:]
 
 
-def note_record_use(records, cam, device):
+def note_record_use(records, cam, device, n=0):
     """After a forward launch that wrote ``records``: queue a 4-byte copy of the pool's bump counter
     (the slots the launch asked for, also beyond the pool's end) to pinned host memory.  Nothing waits
-    for it; the next ``new_records`` of this image size reads it."""
+    for it; the next ``new_records`` of this scene size and image shape on this stream reads it."""
     ntiles, head = _pool_geometry(cam)
-    if records is None or records.numel() < head + 256 + REC_SLOT_WORDS * 4 or records.numel() // 4 // ntiles < REC_LIST_WORDS + REC_SLOT_WORDS:
+    use = _rec_usage.get(_usage_key(cam, device, n))
+    # (the library keeps sample sums only in a record with room for the hit lists and at least one slot per tile)
+    if use is None or records is None or records.numel() // 4 // ntiles < REC_LIST_WORDS + REC_SLOT_WORDS:
         return
-    key = (str(device), cam.width, cam.height)
-    use = _rec_usage.get(key)
-    if use is None:
-        if len(_rec_usage) >= 64:
-            del _rec_usage[next(iter(_rec_usage))]
-        use = _rec_usage[key] = dict(pinned=torch.zeros(1, dtype=torch.int32).pin_memory(), event=torch.cuda.Event(),
-                                     pending=False, need=[])
     use["allocated"] = records.numel()
     _read_record_use(use)
     if use["pending"]:
@@ -307,10 +334,10 @@ def note_record_use(records, cam, device):
     use["pending"] = True
 
 
-def record_use(cam, device):
-    """(bytes allocated for the last record of this image size, bytes of it the last launch read back used:
-    hit-list regions + sample-sum slots), or None before the first launch has reported."""
-    use = _rec_usage.get((str(device), cam.width, cam.height))
+def record_use(cam, device, n=0):
+    """(bytes allocated for the last record of this scene size and image shape on this stream, bytes the last
+    launch read back asked for: hit-list regions + sample-sum slots), or None before the first launch has reported."""
+    use = _rec_usage.get(_usage_key(cam, device, n))
     if use is None:
         return None
     _read_record_use(use)

@@ -113,12 +113,13 @@ class RenderOptixFunction(torch.autograd.Function):
         stale = gas is None or not isinstance(gas, u_ox.AccelerationStructure) or gas.n != n or gas.device != dev
         if stale:
             gas = u_ox.AccelerationStructure(n, dev)
-        if settings.update and not stale:
+        unbuilt = stale or not gas.built      # nothing in the workspace to refit or to reuse
+        if settings.update and not unbuilt:
             # render_optix.py:114-115: the existing structure takes the new boxes and keeps its shape
             if not settings.gas_is_current:
                 boxes, _, _ = u_ox.ellipsoids_bbox_from_quat(normalized_quaternions, positions, scales, densities)
                 u_ox.update_acceleration_structure(gas, boxes)
-        elif stale or not settings.gas_is_current:
+        elif unbuilt or not settings.gas_is_current:
             gas.build_from_gaussians(positions, scales, normalized_quaternions, densities)
         settings.gas = gas
         order_sh = int(round(math.sqrt(color_features.shape[2]))) - 1   # render_optix.py:119
@@ -127,11 +128,12 @@ class RenderOptixFunction(torch.autograd.Function):
                           settings.num_sph_gauss, order_sh)
         prims = u_ox.pack_prims(gas, cam, positions, scales, normalized_quaternions, densities, rgb)
         # when a backward will follow, the forward leaves a record of its hit lists for it to replay
-        records = u_ox.new_records(cam, dev, settings.rec_tile_words) if (any(ctx.needs_input_grad[:8]) and settings.record_hits) else None
+        records = (u_ox.new_records(cam, dev, settings.rec_tile_words, n=n)
+                   if (any(ctx.needs_input_grad[:8]) and settings.record_hits) else None)
         ray_colors = u_ox.march_forward(gas, cam, prims, settings.dt_step, settings.dynamic_sampling,
                                         settings.max_prim_slice, settings.white_background, settings.t_eps,
                                         settings.stats, records)
-        u_ox.note_record_use(records, cam, dev)
+        u_ox.note_record_use(records, cam, dev, n)
         ctx.records = records
         ctx.settings = settings
         ctx.cam = cam

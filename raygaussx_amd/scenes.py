@@ -65,6 +65,12 @@ CONFIGS = {
             max_prim_slice=512, t_eps=1e-4, n_cameras=300),
     4: dict(n=1_000_000, width=1024, height=1024, fov=39.6, dt_step=0.0025, dynamic_sampling=False,
             max_prim_slice=2048, t_eps=1e-3, n_cameras=100),
+    # Not a benchmark configuration: the march kernels' best case, for pricing the implementation apart from a
+    # workload's sparsity.  A few hundred large, faint, isotropic Gaussians in the ball of configuration 4: each covers
+    # hundreds of pixels and a dozen slabs, so all rays of a tile hit the same Gaussians, a ray's chord through a
+    # Gaussian fills whole slabs, no ray saturates, and the tree is a few levels deep.
+    "coherent": dict(n=512, width=800, height=800, fov=39.6, dt_step=0.0025, dynamic_sampling=False,
+                     max_prim_slice=2048, t_eps=1e-3, n_cameras=100),
 }
 
 
@@ -86,7 +92,7 @@ def make_scene(config, n=None, sh_degree=3, device="cpu", seed=None):
     """
     cfg = CONFIGS[config]
     n = cfg["n"] if n is None else n
-    gen = torch.Generator().manual_seed(1234 + (2 if config == 3 else config) if seed is None else seed)
+    gen = torch.Generator().manual_seed(1234 + {3: 2, "coherent": 9}.get(config, config) if seed is None else seed)
     if config == 0:
         pos = torch.rand(n, 3, generator=gen) * 2.0 - 1.0
         log_s = torch.randn(n, 3, generator=gen) * 0.4 - 3.5
@@ -103,11 +109,16 @@ def make_scene(config, n=None, sh_degree=3, device="cpu", seed=None):
     elif config == 4:
         pos = _ball(n, 2.0, gen)
         log_s = torch.randn(n, 3, generator=gen) * 0.5 - 4.5
+    elif config == "coherent":
+        pos = _ball(n, 2.0, gen)
+        log_s = torch.full((n, 3), math.log(0.5))
     else:
         raise ValueError(f"unknown config {config}")
     quat = torch.randn(n, 4, generator=gen)
     quat = quat / quat.norm(dim=1, keepdim=True)
     dens = torch.nn.functional.softplus(torch.randn(n, generator=gen))
+    if config == "coherent":
+        dens = torch.full((n,), 0.15)      # k = sqrt(2 ln 1.5) = 0.9: visible to 0.45 from the centre
     k = (sh_degree + 1) ** 2
     sh = torch.empty(n, 3, k)
     sh[:, :, 0] = torch.randn(n, 3, generator=gen) * 0.2 + 0.5
@@ -127,7 +138,7 @@ def make_camera(config, index=0, width=None, height=None):
     if config == 0:
         r = 4.0 / math.sqrt(3.0)
         eye = (r, r, r)
-    elif config in (1, 4):
+    elif config in (1, 4, "coherent"):
         # golden-angle spiral over the upper hemisphere, radius 4
         m = cfg["n_cameras"]
         z = (index % m + 0.5) / m

@@ -115,3 +115,18 @@ def same_march(orc, ctx, gpu_counts, ids=None):
     _, oc = orc.march_forward_counts(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], ids)
     gc = gpu_counts if ids is None else gpu_counts[ids]
     return (oc == gc).all(1), oc
+
+
+def cutoff_stable_rays(orc, ctx, img, ids=None):
+    """Rays on none of whose samples the cut-off decision of the backward depends on the arrangement of the
+    arithmetic: mask over ``ids``.
+
+    The backward's gradient loop decides ``power < k^2`` per sample.  The reference forms that power in its
+    backward by another arrangement than in its forward (backward/gaussians_aabb.cu:375-396: t0 = tbuffer +
+    0.5 dt, a 3x3 matrix product; forward 112-180: fmaf, dot products); the kernels here use the forward's.
+    One ulp of t moves the power of a thin Gaussian by 1e-4 of its value, so the two disagree on a sample that
+    sits that close to k^2 -- and one sample flipped is, for a few hundred rays, 1e-3 of the whole gradient's
+    norm.  The oracle counts such samples per ray, from its own two arrangements; a ray with one is set aside.
+    Call before ``render_backward`` (which drops the oracle's candidate tree)."""
+    counts = orc.march_backward_in_cut(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], img, ids)
+    return counts[:, 1] == 0

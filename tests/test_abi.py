@@ -86,6 +86,27 @@ def test_bad_arguments_are_rejected_before_any_launch():
         _lib.check(-2)
 
 
+def test_refit_of_an_unbuilt_or_mismatched_structure_is_refused_on_the_host():
+    """update_acceleration_structure walks the tree a build left in the workspace, so the mirror refuses it
+    for a structure that was never built and for anything but one box per Gaussian of that build -- before
+    any launch (the library's own device-side check of the workspace header backs this up)."""
+    gas = u_ox.AccelerationStructure.__new__(u_ox.AccelerationStructure)
+    gas.n, gas.device, gas.built, gas.ws = 100, "cpu", False, torch.zeros(256, dtype=torch.uint8)
+    with pytest.raises(_lib.RgxError, match="never built"):
+        gas.update(torch.zeros(100, 6))
+    with pytest.raises(_lib.RgxError, match="never built"):
+        u_ox.update_acceleration_structure(gas, torch.zeros(100, 6))
+    gas.built = True
+    for bad in (torch.zeros(99, 6), torch.zeros(100, 5), torch.zeros(600)):
+        with pytest.raises(_lib.RgxError, match=r"\(100, 6\)"):
+            gas.update(bad)
+    with pytest.raises(_lib.RgxError, match=r"\(100, 6\)"):
+        gas.build_from_boxes(torch.zeros(101, 6))
+    lib = _lib.lib()
+    null = C.c_void_p(0)
+    assert lib.rgx_refit_aabbs(null, C.c_int64(10), null, C.c_size_t(0), null) == -1
+
+
 def test_missing_library_is_an_error_not_a_fallback(monkeypatch):
     monkeypatch.setattr(_lib, "_lib", None)
     monkeypatch.setattr(_lib, "LIB_PATH", "/nonexistent/librgx.so")
@@ -167,6 +188,8 @@ def test_bench_finds_its_stored_profile_figures():
                           ("c3_3M_1920x1080_fwd", "march_forward")):
         traffic, source = bench.stored_traffic(workload, key)
         assert traffic and traffic > 1e8 and source.startswith("profiles/") and os.path.exists(os.path.join(root, source))
-        issue = bench.valu_issue(workload, key, 7.0)
-        assert issue and issue["instructions_per_launch"] > 1e9 and 0.0 < issue["frac"] < 4.0
+        bench._valu_measured = dict(value=600.0)        # what the probe kernel would measure on the GPU
+        issue = bench.valu_issue(workload, key, 7.0, "cpu")
+        assert issue and issue["instructions_per_launch"] > 1e9 and 0.0 < issue["frac"] <= 1.0 and issue["peak"] == 600.0
+        assert bench.valu_issue(workload, key, 0.01, "cpu")["above_peak"]       # an impossible pairing is flagged, frac capped
     assert bench.stored_traffic("c4_1M_800x800", "no_such_kernel") == (None, None)

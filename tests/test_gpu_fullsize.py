@@ -152,11 +152,13 @@ def test_large_image_of_a_small_scene(gx, orc):
         assert cos >= COS_MIN and rel <= REL_MAX, (k, cos, rel)
 
 
-def _adaptive_gates(gx, orc, sc, cam, cfg, ids, img, st, ctx, dloss):
+def _adaptive_gates(gx, orc, sc, cam, cfg, ids, img, st, ctx, dloss, max_aside=0.03, max_missed=0.01):
     """Image and gradient gates on a ray sample, ray by ray (gpu_common.comparable_rays): rays that
     blended other slabs than on the CPU, or on which the oracle itself jumps when its adaptive step
     moves by a few ulp, are set aside, counted and bounded (none with the fixed step); every other ray
-    must meet the image gate, and the gradient of the loss restricted to them the gradient gates."""
+    must meet the image gate, and the gradient of the loss restricted to them the gradient gates.
+    ``max_aside`` / ``max_missed``: the shares of the sample that may be set aside / may miss the image
+    gate, about twice what the case measures; no ray at all may be further than 5e-3 from the oracle."""
     _, counts = gx.gpu_forward_counts(sc, cam, cfg)
     same, n_rephased, n_edge = gx.comparable_rays(orc, ctx, img, counts, ids)
     _, oc = gx.same_march(orc, ctx, counts, ids)
@@ -171,8 +173,9 @@ def _adaptive_gates(gx, orc, sc, cam, cfg, ids, img, st, ctx, dloss):
               f"{err[same].max():.2e}" + (f", on them {err[~same].max():.2e}" if (~same).any() else ""), flush=True)
         assert oc[:, 1].sum() > 20000
         assert err[same].max() <= IMG_TOL                                       # every comparable ray meets the gate
-        assert (err > IMG_TOL).sum() <= 0.02 * same.size                        # the rays that miss it (all explained) are few
-        assert n_rephased + n_edge <= (0.15 * same.size if cfg["dynamic_sampling"] else 0)
+        assert (err > IMG_TOL).sum() <= max_missed * same.size                  # the rays that miss it (all explained) are few
+        assert n_rephased + n_edge <= (max_aside * same.size if cfg["dynamic_sampling"] else 0)
+        assert err.max() < 5e-3                                                 # no ray, set aside or not, is far off
         if stats:
             assert out["stats_fwd"]["hit_pairs"] == out["stats_bwd"]["hit_pairs"]
         for k in PARAMS:
@@ -202,7 +205,8 @@ def test_heavy_tailed_scene_ray_sample_against_the_oracle(gx, orc):
         cfg = dict(scenes.CONFIGS[2], dynamic_sampling=adaptive)
         img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"], ray_ids=ids)
         _step(f"configs[2] scene, 1 M Gaussians, 1237x822, adaptive step {adaptive}")
-        _adaptive_gates(gx, orc, sc, cam, cfg, ids, img, st, ctx, dloss)
+        # measured with the adaptive step: 1 re-phased + 15 on a cut-off edge of 256 rays (6 %), 1 above the gate
+        _adaptive_gates(gx, orc, sc, cam, cfg, ids, img, st, ctx, dloss, max_aside=0.12, max_missed=0.01)
 
 
 def test_tile_cooperative_and_per_ray_queries_find_the_same_hits(gx, orc, big):
@@ -352,10 +356,11 @@ def test_inference_orbit_3M_gaussians_1080p(gx, orc):
         print(f"camera {index}: of {same.size} rays {n_rephased} re-phased, {n_edge} on a cut-off edge; image max err on the others "
               f"{err[same].max():.2e}" + (f", on them {err[~same].max():.2e}" if (~same).any() else ""), flush=True)
         assert err[same].max() <= IMG_TOL                   # every comparable ray meets the gate
+        assert err.max() < 5e-3                             # no ray, set aside or not, is far off
         missed += int((err > IMG_TOL).sum())
         rephased += n_rephased + n_edge
         total += same.size
-    assert missed <= 0.02 * total and rephased <= 0.15 * total
+    assert missed <= 0.01 * total and rephased <= 0.03 * total      # measured: 0 and 3 of 480 rays
 
 
 def test_heavy_tailed_scene_at_3M_gaussians(gx, orc):
@@ -431,3 +436,163 @@ def test_accumulation_window_perturb_and_rebuild_at_1M(gx, orc):
         cos, rel = gx.cos_rel(got[k], want[k])
         print(f"window 2 {k}: 1 - cos {1 - cos:.2e}, rel {rel:.2e}", flush=True)
         assert cos >= COS_MIN and rel <= REL_MAX, (k, cos, rel)
+
+
+def test_object_scene_300k_gaussians_800x800(gx, orc):
+    """The object-centric configuration at its own size: 300 000 Gaussians in the unit ball, 800x800, three
+    cameras of its 100-camera hemisphere.  The densest regime per slab (some 15 hits per ray and slab, most
+    rays missing the object).  Forward and backward against the oracle on a ray sample (its culled candidate
+    search), through the counting kernels and through the ones a training loop launches; per-ray march
+    counters equal the oracle's; the forward repeats bit for bit."""
+    n, w, h = 300_000, 800, 800
+    cfg = scenes.CONFIGS[1]
+    assert (cfg["n"], cfg["width"], cfg["height"]) == (n, w, h) and not cfg["dynamic_sampling"]
+    sc = scenes.scene_to_numpy(scenes.make_scene(1))
+    sc = {k: sc[k] for k in PARAMS}
+    assert sc["positions"].shape[0] == n
+    for index in (0, 37, 81):
+        cam = scenes.make_camera(1, index)
+        rng = np.random.default_rng(50 + index)
+        ids = np.unique(rng.integers(0, w * h, 512))
+        img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], False, cfg["max_prim_slice"], ray_ids=ids, cull=True)
+        _, oc = orc.march_forward_counts(ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"], ids)
+        # Rays that hold a sample on which the reference's forward and backward arrangements of `power < k^2`
+        # disagree (gpu_common.cutoff_stable_rays; 1, 3 and 0 of 512 here) are left out of the loss that faces
+        # the reference's backward; with them in, the gradients face the oracle deciding by the forward's
+        # arrangement, as the kernels do -- all else as the reference has it.
+        stable = gx.cutoff_stable_rays(orc, ctx, img, ids)
+        assert (~stable).sum() <= 0.02 * len(ids)
+        dloss = np.zeros((w * h, 3), np.float32)
+        dloss[ids] = rng.normal(size=(len(ids), 3)).astype(np.float32)
+        dl = np.zeros_like(dloss)
+        dl[ids[stable]] = dloss[ids[stable]]
+        orc.set_backward_mask_form(1)
+        try:
+            og_all, _ = orc.render_backward(sc, dict(ctx, cull=False), img, dloss)      # (keeps the candidate tree)
+        finally:
+            orc.set_backward_mask_form(0)
+        og, _ = orc.render_backward(sc, ctx, img, dl)
+        assert st["hit_pairs"] > 40000 and st["overflow_rays"] == 0
+        _step(f"configs[1]: 300 k Gaussians, 800x800, camera {index}, {int((~stable).sum())} rays on a cut-off edge")
+        _, counts = gx.gpu_forward_counts(sc, cam, cfg)
+        assert np.array_equal(counts[ids], oc)                  # slabs blended and hit-list lengths, ray by ray
+        images = []
+        for stats in (True, False):
+            out = gx.gpu_render(sc, cam, cfg, want_grad=dl, stats=stats)
+            images.append(out["image"])
+            err = np.abs(out["image"][ids] - img[ids]).max()
+            print(f"camera {index}, stats {stats}: image max err {err:.2e}", flush=True)
+            assert err <= IMG_TOL
+            if stats:
+                assert out["stats_fwd"]["hit_pairs"] == out["stats_bwd"]["hit_pairs"] > 3e7
+                assert out["stats_fwd"]["slabs"] == out["stats_bwd"]["slabs"]
+                assert out["stats_fwd"]["overflow_rays"] == 0 and out["stats_bwd"]["replay_lost"] == 0
+            for k in PARAMS:
+                cos, rel = gx.cos_rel(out["grads"][k], og[k])
+                print(f"camera {index}, stats {stats}, {k}: 1 - cos {1 - cos:.2e}, rel {rel:.2e}", flush=True)
+                assert cos >= COS_MIN and rel <= REL_MAX, (index, stats, k, cos, rel)
+            full = gx.gpu_render(sc, cam, cfg, want_grad=dloss, stats=stats)
+            for k in PARAMS:
+                cos, rel = gx.cos_rel(full["grads"][k], og_all[k])
+                print(f"camera {index}, stats {stats}, all rays, {k}: 1 - cos {1 - cos:.2e}, rel {rel:.2e}", flush=True)
+                assert cos >= COS_MIN and rel <= REL_MAX, (index, stats, "all rays", k, cos, rel)
+        assert np.array_equal(images[0], images[1])             # counting or not: the same image, bit for bit
+        # the forward that records nothing (no gradient wanted) collects crowded slabs half by half, which
+        # changes the order of the sample sums, not the hits: equal to rounding, and repeatable bit for bit
+        plain = [gx.gpu_render(sc, cam, cfg, stats=False)["image"] for _ in range(2)]
+        assert np.array_equal(plain[0], plain[1])
+        assert np.abs(plain[0] - images[1]).max() <= 2e-6
+        assert np.abs(plain[0][ids] - img[ids]).max() <= IMG_TOL
+        # most rays of this configuration miss the object and keep the background
+        assert 0.3 < np.all(images[0] == 1.0, axis=1).mean() < 0.8
+
+
+@pytest.mark.timeout(600)
+def test_training_stress_1M_1024x1024_windows_with_reorder_and_rebuild(gx, orc):
+    """The training-step stress configuration as stated: 1 M Gaussians at 1024x1024, gradients accumulated
+    over the 20 views of a window (one tree, marked current for views 2..20), the centres then perturbed by
+    N(0, 1e-3), the Gaussians put in Morton order -- every parameter gathered with the one permutation, as
+    classes/point_cloud.py:1017-1046 does every 1000 iterations -- and a second window that rebuilds the tree
+    in place over the renumbered Gaussians.  Accumulated gradients of both windows against the sum of the
+    oracle's per-view gradients on ray samples, the second window's in the new numbering; renumbering must
+    not change the image."""
+    from raygaussx_amd.render_optix import RenderOptixFunction, default_settings
+    from raygaussx_amd.reordering import morton_order, reorder_tensors
+    w = h = 1024
+    cfg = scenes.CONFIGS[4]
+    assert (cfg["n"], cfg["width"], cfg["height"]) == (N, w, h)
+    sc = scenes.scene_to_numpy(scenes.make_scene(4))
+    sc = {k: sc[k] for k in PARAMS}
+    rng = np.random.default_rng(61)
+    empty = (torch.zeros(N, 3, 0, device=gx.DEV), torch.zeros(N, 0, device=gx.DEV), torch.zeros(N, 0, 3, device=gx.DEV))
+
+    def window(params, scene, cams, gas, n_rays):
+        """20 views accumulate in .grad of ``params`` (device leaves); ``scene``: the same values for the oracle."""
+        want = {k: np.zeros(scene[k].shape, np.float64) for k in PARAMS}
+        worst, first = 0.0, None
+        for i, ci in enumerate(cams):
+            cam = scenes.make_camera(4, ci, width=w, height=h)
+            ids = np.sort(rng.choice(w * h, n_rays, replace=False)).astype(np.int64)
+            dloss = np.zeros((w * h, 3), np.float32)
+            dloss[ids] = rng.normal(size=(n_rays, 3)).astype(np.float32)
+            s = default_settings(cam.to(gx.DEV), cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"], gas=gas)
+            s.gas_is_current = i > 0
+            img = RenderOptixFunction.apply(*params, *empty, s)
+            img.backward(torch.from_numpy(dloss).to(gx.DEV))
+            gas = s.gas
+            if first is None:
+                first = img.detach().cpu().numpy()
+            o_img, _, ctx = orc.render_forward(scene, cam, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"],
+                                               ray_ids=ids, cull=True)
+            og, _ = orc.render_backward(scene, ctx, o_img, dloss)
+            worst = max(worst, float(np.abs(img.detach().cpu().numpy()[ids] - o_img[ids]).max()))
+            for k in PARAMS:
+                want[k] += og[k]
+        torch.cuda.synchronize()
+        return {k: p.grad.cpu().numpy() for k, p in zip(PARAMS, params)}, want, worst, gas, first
+
+    def gates(label, got, want):
+        for k in PARAMS:
+            cos, rel = gx.cos_rel(got[k], want[k])
+            print(f"{label} {k}: 1 - cos {1 - cos:.2e}, rel {rel:.2e}", flush=True)
+            assert cos >= COS_MIN and rel <= REL_MAX, (label, k, cos, rel)
+
+    _step("configs[4] at 1024x1024: window of 20 views, one tree")
+    params = [torch.from_numpy(sc[k]).to(gx.DEV).requires_grad_(True) for k in PARAMS]
+    got, want, worst, gas, _ = window(params, sc, list(range(20)), None, 24)
+    assert worst <= IMG_TOL
+    gates("window 1", got, want)
+
+    # the optimiser step's effect on the centres, then the periodic reordering along the z-order curve
+    _step("perturbation N(0, 1e-3) of the centres, Morton order, one gather for all parameters")
+    with torch.no_grad():
+        moved = [p.detach().clone() for p in params]
+        moved[0] += torch.from_numpy(rng.normal(size=sc["positions"].shape).astype(np.float32) * 1e-3).to(gx.DEV)
+        unordered = {k: t.cpu().numpy() for k, t in zip(PARAMS, moved)}
+        order = morton_order(moved[0])
+        moved = reorder_tensors(order, moved)
+    order_np = order.cpu().numpy()
+    assert np.array_equal(np.sort(order_np), np.arange(N))
+    scene2 = {k: t.cpu().numpy() for k, t in zip(PARAMS, moved)}
+    for k in PARAMS:
+        assert np.array_equal(scene2[k], unordered[k][order_np])            # the gather is t[order] for every tensor
+    codes = orc.morton_codes(scene2["positions"])
+    assert np.all(np.diff(codes.astype(np.int64)) >= 0)                     # and leaves the cloud sorted along the curve
+    params2 = [t.requires_grad_(True) for t in moved]
+
+    _step("configs[4] at 1024x1024: second window, tree rebuilt in place over the renumbered Gaussians")
+    ws_before = gas.ws.data_ptr()
+    got2, want2, worst2, gas2, first2 = window(params2, scene2, list(range(20, 40)), gas, 24)
+    assert gas2 is gas and gas.ws.data_ptr() == ws_before and worst2 <= IMG_TOL
+    gates("window 2", got2, want2)
+    # renumbering changes neither the image nor, up to the permutation, the gradients: camera 20 on the
+    # perturbed scene in its old numbering
+    _step("camera 20 on the perturbed scene before the renumbering")
+    cam = scenes.make_camera(4, 20, width=w, height=h)
+    g = rng.normal(size=(w * h, 3)).astype(np.float32)
+    a = gx.gpu_render(unordered, cam, cfg, want_grad=g, stats=False)
+    b = gx.gpu_render(scene2, cam, cfg, want_grad=g, stats=False)
+    assert np.abs(a["image"] - first2).max() <= 2e-6 and np.abs(b["image"] - first2).max() <= 2e-6
+    for k in PARAMS:
+        cos, rel = gx.cos_rel(b["grads"][k], a["grads"][k][order_np])
+        assert cos >= 1 - 1e-6 and rel <= 1e-4, (k, cos, rel)

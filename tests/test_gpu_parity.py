@@ -392,8 +392,9 @@ def test_dynamic_sampling_lobes_supersampling_black_background(gx, orc):
     print(f"of {same.size} rays: {n_rephased} re-phased, {n_edge} on a cut-off edge; image max err on the others {err[same].max():.2e}, "
           f"on them {err[~same].max() if (~same).any() else 0.0:.2e}", flush=True)
     assert err[same].max() <= IMG_TOL                     # every comparable ray meets the gate
-    assert (err > IMG_TOL).sum() <= 0.01 * same.size      # and the rays that miss it (all explained) are few
-    assert n_rephased + n_edge <= 0.15 * same.size
+    assert (err > IMG_TOL).sum() <= 0.005 * same.size     # the rays that miss it (all explained) are few: 1 of 2 790 measured
+    assert n_rephased + n_edge <= 0.03 * same.size        # measured: 0 re-phased + 31 on an edge of 2 790 (1.1 %)
+    assert err.max() < 5e-3                               # and no ray, set aside or not, is far off
     dl = dloss * same[:, None]
     og, _ = orc.render_backward(sc, ctx, img, dl)
     out = gx.gpu_render(sc, cam, cfg, white=False, supersampling=(2, 1), want_grad=dl)

@@ -73,28 +73,51 @@ VALU_NOMINAL_GINST = 256 * 4 * 2.4 / 4.0
 _valu_measured = None
 
 
+PROBE_KINDS = ("v_fma_f32", "v_add_f32", "v_mov_b32", "v_and_b32", "v_cmp_lt_f32", "v_cndmask_b32", "v_max_f32",
+               "v_add_f32_dpp", "v_lshlrev_b32", "v_exp_f32")
+
+
+def probe_rate(dev, kind, waves_per_simd, iters=1024, reps=5):
+    """(G wave instructions/s, launch ms, instructions) of rgx_probe_valu_rate: one instruction class, sixteen
+    independent registers per lane, ``waves_per_simd`` wavefronts on each of the 1024 SIMDs; best of ``reps``."""
+    sink = torch.zeros(4, device=dev)
+    count = C.c_uint64(0)
+    best = float("inf")
+    for rep in range(reps + 2):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        L.check(L.lib().rgx_probe_valu_rate(C.c_int32(256 * 4 * waves_per_simd), C.c_int32(iters), C.c_int32(kind), L.ptr(sink),
+                                            C.byref(count), L.stream(dev)))
+        b.record()
+        torch.cuda.synchronize()
+        if rep >= 2:
+            best = min(best, a.elapsed_time(b))
+    return count.value / (best * 1e-3) / 1e9, best, count.value
+
+
 def valu_measured(dev):
-    """G VALU wave instructions per second this card issues, measured: a kernel of independent fp32
-    multiply-adds (rgx_probe_valu_rate: 8 wavefronts per SIMD, nothing but v_fma_f32 and a loop counter), its
-    instruction count known from its shape, timed with events on the launch stream; best of five launches."""
+    """G VALU wave instructions per second this card issues, measured: independent v_fma_f32 (rgx_probe_valu_rate,
+    8 wavefronts per SIMD, nothing but the multiply-adds and a loop counter), the instruction count known from the
+    kernel's shape, timed with events on the launch stream.  Also at the three wavefronts per SIMD the march kernels
+    run with, and for a compare (the slower class of VALU instruction: compares, selects, min / max, DPP, shifts)."""
     global _valu_measured
     if _valu_measured is None:
-        sink = torch.zeros(4, device=dev)
-        count = C.c_uint64(0)
-        waves, iters = 256 * 4 * 8, 2048
-        best = float("inf")
-        for rep in range(7):
-            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            L.check(L.lib().rgx_probe_valu_rate(C.c_int32(waves), C.c_int32(iters), L.ptr(sink), C.byref(count), L.stream(dev)))
-            b.record()
-            torch.cuda.synchronize()
-            if rep >= 2:
-                best = min(best, a.elapsed_time(b))
-        _valu_measured = dict(value=round(count.value / (best * 1e-3) / 1e9, 1), unit="G wave instructions/s",
-                              nominal=round(VALU_NOMINAL_GINST, 1), instructions=count.value, kernel_ms=round(best, 4),
-                              what="independent v_fma_f32 chains, 8 wavefronts per SIMD")
+        rate, ms, count = probe_rate(dev, 0, 8, iters=2048)
+        _valu_measured = dict(value=round(rate, 1), unit="G wave instructions/s", nominal=round(VALU_NOMINAL_GINST, 1),
+                              instructions=count, kernel_ms=round(ms, 4), what="independent v_fma_f32, 8 wavefronts per SIMD",
+                              fma_at_3_waves_per_simd=round(probe_rate(dev, 0, 3)[0], 1),
+                              cmp_at_3_waves_per_simd=round(probe_rate(dev, 4, 3)[0], 1),
+                              exp_at_3_waves_per_simd=round(probe_rate(dev, 9, 3)[0], 1))
     return _valu_measured
+
+
+def valu_cost_table(dev):
+    """Clocks per wave instruction and SIMD (1024 SIMDs at 2.4 GHz over the measured rate) of every probe kind at
+    1, 2, 3, 4 and 8 wavefronts per SIMD."""
+    table = {}
+    for kind, name in enumerate(PROBE_KINDS):
+        table[name] = {str(w): round(1024 * 2.4 / probe_rate(dev, kind, w, reps=3)[0], 2) for w in (1, 2, 3, 4, 8)}
+    return table
 
 
 def valu_issue(workload, kernel_key, kernel_ms, dev):
@@ -367,6 +390,7 @@ def training_leg(dev, workload, steps, warmup, opts, in_flight=1):
         s.record_hits = not opts.no_records
         if opts.rec_tile_words is not None:
             s.rec_tile_words = opts.rec_tile_words
+        s.rec_half_sums = opts.half_sums
         img = RenderOptixFunction.apply(*params, s)
         gas = s.gas
         if not forward_only:
@@ -397,6 +421,12 @@ def training_leg(dev, workload, steps, warmup, opts, in_flight=1):
     timing = L.timing_read()
     L.timing_enable(False)
     sections = read_sections() if opts.sections else None
+    if opts.sections and opts.dump_tile_times:
+        # per workgroup (launch order): cycles per section, waves, kernel, start and end of its last wave (100 MHz ticks)
+        rows = np.zeros((2, 65536, 16), np.uint32)
+        L.check(L.lib().rgx_debug_section_rows(rows.ctypes.data_as(C.c_void_p)))
+        used = int(max(np.nonzero(rows[:, :, 12].sum(0))[0], default=0)) + 1
+        np.save(opts.dump_tile_times, rows[:, :used])
     steady_peak = torch.cuda.max_memory_allocated(dev)
     for i in range(steps):     # census: the same views once more, counted, not timed
         step(warmup + i, census=True)
@@ -429,7 +459,7 @@ def training_leg(dev, workload, steps, warmup, opts, in_flight=1):
     if not forward_only:
         cand.append(("march_backward", bwd_name, (64.0 + 56.0) * hits_per_launch + 24.0 * n_rays))
     per_kernel = {}
-    default_record = not (opts.no_records or opts.rec_tile_words is not None)
+    default_record = not (opts.no_records or opts.rec_tile_words is not None or opts.half_sums)
     for key, name, nbytes in cand:
         ms, cnt = timing[key]
         avg = ms / max(cnt, 1)
@@ -478,7 +508,7 @@ def training_leg(dev, workload, steps, warmup, opts, in_flight=1):
     out["views_in_flight"] = flight
     if sections is not None:
         out["sections"] = sections
-    rec_use = None if forward_only else u_ox.record_use(cam_structs[0], dev, n)
+    rec_use = None if forward_only else u_ox.record_use(cam_structs[0], dev, n, 1 if opts.half_sums else 0)
     out["memory"] = dict(first_view_peak_GB=round(first_peak / 1e9, 3), steady_peak_GB=round(steady_peak / 1e9, 3),
                          first_over_steady=round(first_peak / max(steady_peak, 1), 3),
                          resident_before_GB=round(base_mem / 1e9, 3),
@@ -512,12 +542,17 @@ def main():
     ap.add_argument("--rec-tile-words", type=int, default=None,
                     help="record size per tile in 32-bit words (16384: hit lists only, no per-sample sums); "
                          "default: the renderer's own")
+    ap.add_argument("--half-sums", action="store_true",
+                    help="the record keeps the per-sample colour sums in half precision (settings.rec_half_sums)")
     ap.add_argument("--in-flight", type=int, default=2,
                     help="after the timed steps, time the same steps again with this many views in flight, each on "
                          "a stream of its own (reported beside the headline figure; 1 = skip)")
     ap.add_argument("--sections", action="store_true",
                     help="also report the march kernels' per-section cycle census; needs the diagnostic build "
                          "(python -m raygaussx_amd.build --sections; RGX_LIB_PATH=raygaussx_amd/librgx_sections.so)")
+    ap.add_argument("--dump-tile-times", default=None,
+                    help="with --sections: write the per-workgroup table of the timed steps (cycles per section, start and "
+                         "end of the workgroup's last wave) to this .npy file")
     ap.add_argument("--side-kernels", action="store_true",
                     help="time the entry points around the march (image epilogue, reorder gather, distCUDA2, viewer launch) "
                          "instead of the training step; one JSON line")
@@ -542,7 +577,7 @@ def main():
         return
     L.lib()
     if args.calibrate_valu:
-        print(json.dumps(dict(calibration="valu", launches=7, **valu_measured(dev))))
+        print(json.dumps(dict(calibration="valu", **valu_measured(dev), clocks_per_instruction_per_simd=valu_cost_table(dev))))
         return
     if args.side_kernels:
         print(json.dumps(side_kernels(dev, args.steps)), flush=True)

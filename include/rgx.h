@@ -59,6 +59,10 @@ typedef struct RgxMarch {
     int32_t max_prim_slice;
     int32_t white_background;
     float t_eps;
+    int32_t record_format; /* of the sample sums a forward leaves in its record for the backward (not in the
+                              reference, which keeps no record): 0 float colour sums, 32 KiB per slab iteration of a
+                              tile; 1 half-precision colour sums with a power-of-two scale per ray and 16 samples,
+                              20.5 KiB.  The forward and the backward of a view must be given the same value. */
 } RgxMarch;
 
 /* Optional device-side counters, accumulated (not reset) by the march kernels. */
@@ -311,14 +315,16 @@ int rgx_collect_tiles(const void *ws, const RgxCamera *cam, const float *prims, 
  * (2^-46 <= |a|, |b| <= 2^46). */
 int rgx_check_plain_arith(const float *a, const float *b, int64_t n, uint32_t *bad, void *stream);
 
-/* Measurement hook (no counterpart in the reference): a kernel of nothing but independent fp32
- * multiply-adds, for the rate at which this card issues VALU instructions -- the ceiling the march
- * kernels, which are bound by instruction issue, are priced against.  Launches `waves` wavefronts
- * (rounded up to whole workgroups of four) that each issue iters * 64 multiply-adds; *instructions
- * (host) receives the number of VALU wave instructions the launch issues in its loops.  `sink`
- * (device, at least one float) keeps the compiler from dropping the arithmetic; nothing is written
- * to it for finite inputs.  The caller times the launch with events on `stream`. */
-int rgx_probe_valu_rate(int32_t waves, int32_t iters, float *sink, uint64_t *instructions, void *stream);
+/* Measurement hook (no counterpart in the reference): a kernel that issues one VALU instruction over
+ * and over on independent registers, for the rate at which this card issues that class of instruction
+ * -- the ceiling the march kernels, which are bound by instruction issue, are priced against.
+ * kind: 0 v_fma_f32, 1 v_add_f32, 2 v_mov_b32, 3 v_and_b32, 4 v_cmp_lt_f32, 5 v_cndmask_b32,
+ * 6 v_max_f32, 7 v_add_f32 with a DPP operand, 8 v_lshlrev_b32, 9 v_exp_f32.  Launches `waves`
+ * wavefronts (rounded up to whole workgroups of four) that each issue iters * 64 of them;
+ * *instructions (host) receives the number of wave instructions the launch issues in its loops.
+ * `sink` (device, at least one float) keeps the registers live; nothing is written to it for finite
+ * inputs.  The caller times the launch with events on `stream`. */
+int rgx_probe_valu_rate(int32_t waves, int32_t iters, int32_t kind, float *sink, uint64_t *instructions, void *stream);
 
 /* ---- Morton reordering of the point cloud --------------------------------- */
 

@@ -25,7 +25,7 @@ class RgxCamera(C.Structure):
 
 class RgxMarch(C.Structure):
     _fields_ = [("dt_step", C.c_float), ("dynamic_sampling", C.c_int32), ("max_prim_slice", C.c_int32),
-                ("white_background", C.c_int32), ("t_eps", C.c_float)]
+                ("white_background", C.c_int32), ("t_eps", C.c_float), ("record_format", C.c_int32)]
 
 
 STATS_FIELDS = ("hit_pairs", "slabs", "empty_slabs", "overflow_rays", "rays_hit", "nodes_visited", "candidates",

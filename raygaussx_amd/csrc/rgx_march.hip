@@ -78,6 +78,7 @@ struct MarchParams {
     float4 *sum_pool;       // sample-sum slots of the record (RGX_SUM_SLOT_WORDS each), or null
     uint32_t *sum_next;     // next free slot (bump counter in the record's pool header)
     int32_t sum_slots;      // slots in the pool
+    int32_t sum_slot_words; // words per slot: RGX_SUM_SLOT_WORDS, or RGX_SUM_SLOT_WORDS_HALF with half-precision colour sums
     uint32_t *faults;       // march workspace: [0] replays that lost their record, [1] sweeps that dropped nodes; or null
     uint32_t *ray_counts;   // counting forward only: per ray, slabs blended and the sum of their hit-list lengths; or null
 };
@@ -93,7 +94,8 @@ enum { RGX_SEC_SWEEP = 0, RGX_SEC_FILTER = 1, RGX_SEC_SHADE = 2, RGX_SEC_LISTS =
        RGX_SEC_SETUP = 6, RGX_SEC_TOP = 7, RGX_SEC_END = 8, RGX_SEC_EPILOGUE = 9, RGX_SEC_WALK = 10, RGX_SEC_FLUSH = 11 };
 enum { RGX_SECK_FWD_RECORD = 0, RGX_SECK_FWD_PLAIN = 1, RGX_SECK_BWD_SUMS = 2, RGX_SECK_BWD_LISTS = 3, RGX_SECK_BWD_TREE = 4, RGX_NSECK = 5 };
 #define RGX_SEC_ROWS 65536 // workgroups per launch the table has rows for (a 1920x1080 launch has 33 024)
-// [forward / backward][workgroup][section]; word RGX_NSEC of a row counts the waves that used it, the next word names their kernel.
+// [forward / backward][workgroup][section]; word RGX_NSEC of a row counts the waves that used it, the next word names their
+// kernel, words 14 and 15 are the start and end of the last wave that used it on the 100 MHz wall clock.
 // The sums live in memory, not in registers: the march kernels have no registers to spare, and a census that made them
 // spill would time another kernel.
 __device__ unsigned g_section_cycles[2][RGX_SEC_ROWS][16];
@@ -103,6 +105,7 @@ struct SectionClock {
     __device__ __forceinline__ void start(int pass)
     {
         row = blockIdx.x < RGX_SEC_ROWS ? g_section_cycles[pass][blockIdx.x] : nullptr;
+        if (threadIdx.x == 0 && row) row[14] = (unsigned)wall_clock64(); // when the wave started, 100 MHz ticks (the last launch's)
         last = (unsigned)__builtin_readcyclecounter();
     }
     __device__ __forceinline__ void to(int k)
@@ -116,6 +119,7 @@ struct SectionClock {
         if (threadIdx.x != 0 || !row) return;
         atomicAdd(row + RGX_NSEC, 1u);
         row[RGX_NSEC + 1] = (unsigned)kernel;
+        row[15] = (unsigned)wall_clock64(); // and when it ended
     }
 };
 struct NoSectionClock {
@@ -1059,6 +1063,13 @@ __device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds 
 // bump counter; a tile that found the pool empty is marked lists-only (status 0).
 #define RGX_REC_LIST_WORDS 16384   // hit-list words per tile when the record also holds sample sums
 #define RGX_SUM_SLOT_WORDS 8192    // 32 samples x 64 rays x 4 words
+// With RgxMarch::record_format 1 a slot keeps the colour sums in half precision: the density sums as before
+// ([32 samples][64 rays] floats: the transmittance must replay bit for bit), then per chunk of 16 samples and ray
+// the 48 colour sums divided by a power of two that brings the largest to [1/2, 1) and rounded to binary16, two to a
+// word ([2 chunks][24 words][64 rays]), then that power of two per chunk and ray ([2][64] floats).  The scale makes
+// the format safe for any density (plain binary16 overflows at 65504); the sums keep 11 bits relative to each
+// value down to 2^-14 of the chunk's largest.
+#define RGX_SUM_SLOT_WORDS_HALF (2048 + 2 * 24 * 64 + 2 * 64)
 #define RGX_REC_COMPLETE 0u        // word 0 of a tile: hit lists complete
 #define RGX_REC_OVERFLOWED 1u      //   the region overflowed (record unusable)
 #define RGX_REC_COMPLETE_SUMS 2u   //   hit lists and sample sums complete
@@ -1071,7 +1082,8 @@ __device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds 
 // tile instead of following indices that mean nothing in its own tables.
 __device__ __forceinline__ uint32_t record_mark(const MarchParams &P, int which)
 {
-    return which == 0 ? (uint32_t)P.n : ((uint32_t)P.cam.width << 16 ^ (uint32_t)P.cam.height ^ __float_as_uint(P.m.dt_step));
+    return which == 0 ? (uint32_t)P.n ^ ((uint32_t)P.m.record_format << 31)
+                      : ((uint32_t)P.cam.width << 16 ^ (uint32_t)P.cam.height ^ __float_as_uint(P.m.dt_step));
 }
 // Status of a tile's record if it is this launch's and complete, else RGX_REC_OVERFLOWED.
 __device__ __forceinline__ uint32_t record_status(const MarchParams &P, const uint32_t *reg)
@@ -1610,7 +1622,7 @@ struct Replayer {
                     mid(false);
                     return false;
                 }
-                body_a(P.sum_pool + (int64_t)(slot1 - 1u) * (RGX_SUM_SLOT_WORDS / 4));
+                body_a(P.sum_pool + (int64_t)(slot1 - 1u) * (P.sum_slot_words / 4));
             }
         } else {
             for (int a = start; a < end;) {
@@ -1674,9 +1686,10 @@ __device__ __forceinline__ uint8_t quantize8(float x)
 // colorBlendingT_chunked (182-203).  VIEWER: the interactive viewer's variant of the same march
 // (cuda_gui/gaussians_aabb.cu): black background, uchar4 colours, and the expected depth
 // sum T (1 - w) t over the samples (its colorBlendingT_chunked, 183-205).
-template <bool RECORD, bool VIEWER, bool STATS>
+template <bool RECORD, bool VIEWER, bool STATS, bool HALF = false>
 __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchParams P)
 {
+    static_assert(RECORD || !HALF, "the colour sums' format is a property of the record");
     RGX_TILE_LDS();
     int px0, py0, tile;
     if (!tile_origin(P, px0, py0, &tile)) return; // whole wave
@@ -1757,16 +1770,38 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_fwd(const MarchPara
             auto keep_sums = [&](int first_sample) {
                 if constexpr (RECORD) {
                     if (rec.slot >= 0) {
-                        float *slot = (float *)(P.sum_pool + (int64_t)rec.slot * (RGX_SUM_SLOT_WORDS / 4));
+                        float *slot = (float *)(P.sum_pool + (int64_t)rec.slot * (P.sum_slot_words / 4));
                         float *dens = slot + first_sample * 64 + threadIdx.x;
-                        float *col = slot + RGX_BUFFER_SIZE * 64 + (first_sample * 64 + threadIdx.x) * 3;
+                        if constexpr (!HALF) {
+                            float *col = slot + RGX_BUFFER_SIZE * 64 + (first_sample * 64 + threadIdx.x) * 3;
 #pragma unroll
-                        for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
-                            // written once, read once by the backward: keep them out of the caches' way
-                            __builtin_nontemporal_store(sg[i], dens + i * 64);
-                            __builtin_nontemporal_store(cr[i], col + i * 192);
-                            __builtin_nontemporal_store(cg[i], col + i * 192 + 1);
-                            __builtin_nontemporal_store(cb[i], col + i * 192 + 2);
+                            for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
+                                // written once, read once by the backward: keep them out of the caches' way
+                                __builtin_nontemporal_store(sg[i], dens + i * 64);
+                                __builtin_nontemporal_store(cr[i], col + i * 192);
+                                __builtin_nontemporal_store(cg[i], col + i * 192 + 1);
+                                __builtin_nontemporal_store(cb[i], col + i * 192 + 2);
+                            }
+                        } else {
+                            const int chunk = first_sample / RGX_CHUNK_SIZE;
+                            float big = 0.f;
+#pragma unroll
+                            for (int i = 0; i < RGX_CHUNK_SIZE; ++i) {
+                                __builtin_nontemporal_store(sg[i], dens + i * 64);
+                                big = fmaxf(big, fmaxf(fabsf(cr[i]), fmaxf(fabsf(cg[i]), fabsf(cb[i]))));
+                            }
+                            // big = f * 2^e with f in [1/2, 1): everything times 2^-e lies in (-1, 1)
+                            const int e = big > 0.f ? __builtin_amdgcn_frexp_expf(big) : 0;
+                            const float down = __builtin_amdgcn_ldexpf(1.0f, -e);
+                            uint32_t *col = (uint32_t *)slot + RGX_BUFFER_SIZE * 64 + chunk * (24 * 64) + threadIdx.x;
+                            auto value = [&](int k) { return (k % 3 == 0 ? cr[k / 3] : k % 3 == 1 ? cg[k / 3] : cb[k / 3]) * down; };
+#pragma unroll
+                            for (int j = 0; j < 24; ++j) {
+                                const __half2 two = __floats2half2_rn(value(2 * j), value(2 * j + 1));
+                                __builtin_nontemporal_store(*(const uint32_t *)&two, col + j * 64);
+                            }
+                            __builtin_nontemporal_store(__builtin_amdgcn_ldexpf(1.0f, e),
+                                                        slot + RGX_BUFFER_SIZE * 64 + 2 * 24 * 64 + chunk * 64 + threadIdx.x);
                         }
                     }
                 }
@@ -1862,16 +1897,18 @@ __device__ __forceinline__ float group_sum(float v)
 // is the mask the forward blended with.  Per Gaussian the moments turn into 13 sums in its whitened
 // frame (RGX_NSUM); those are summed over the 16 rays of a row with DPP adds and carried on by one
 // lane per row; the change of variables to the 14 gradient words comes after all sums.
-template <bool REPLAY, bool SUMS, bool STATS>
+template <bool REPLAY, bool SUMS, bool STATS, bool HALF = false>
 __device__ __forceinline__ void march_bwd(const MarchParams &P)
 {
     static_assert(REPLAY || !SUMS, "sample sums come with a record");
+    static_assert(SUMS || !HALF, "the colour sums' format is a property of the sample sums");
     int px0, py0, tile;
     if (!tile_origin(P, px0, py0, &tile)) return; // whole wave
     const uint32_t *reg = P.records ? P.records + (int64_t)tile * P.rec_tile_words : nullptr;
     if (REPLAY) {
         // overflowed, not this launch's, or with / without sample sums: another kernel handles the tile
         if (record_status(P, reg) != (SUMS ? RGX_REC_COMPLETE_SUMS : RGX_REC_COMPLETE)) return;
+        if (SUMS && HALF != (P.m.record_format == 1)) return; // (the launcher picks the variant of the record's format)
     } else if (P.only_overflow) {
         if (record_usable(P, reg)) return; // replayed
     }
@@ -1944,20 +1981,33 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
             auto load_sums = [&](const float4 *slot) {
                 RGX_SEC(cn, RGX_SEC_WALK);
                 const float *dens = (const float *)slot + lane;
-                const float *col = (const float *)slot + RGX_BUFFER_SIZE * 64 + lane * 3;
 #pragma unroll
                 for (int i = 0; i < RGX_BUFFER_SIZE; ++i) PA[i] = __builtin_nontemporal_load(dens + i * 64);
-#ifdef RGX_PROBE_FP16_SUMS
-                // probe: what half-precision storage of the colour sums would cost in accuracy (values rounded to
-                // binary16 and back; the density sums stay exact, the transmittance must replay bit for bit)
-                auto h16 = [](float v) { return __half2float(__float2half(v)); };
-#else
-                auto h16 = [](float v) { return v; };
-#endif
+                if constexpr (!HALF) {
+                    const float *col = (const float *)slot + RGX_BUFFER_SIZE * 64 + lane * 3;
 #pragma unroll
-                for (int i = 0; i < RGX_BUFFER_SIZE; ++i)
-                    PB[i] = fmaf(g.x, h16(__builtin_nontemporal_load(col + i * 192)),
-                                 fmaf(g.y, h16(__builtin_nontemporal_load(col + i * 192 + 1)), g.z * h16(__builtin_nontemporal_load(col + i * 192 + 2))));
+                    for (int i = 0; i < RGX_BUFFER_SIZE; ++i)
+                        PB[i] = fmaf(g.x, __builtin_nontemporal_load(col + i * 192),
+                                     fmaf(g.y, __builtin_nontemporal_load(col + i * 192 + 1), g.z * __builtin_nontemporal_load(col + i * 192 + 2)));
+                } else {
+#pragma unroll
+                    for (int chunk = 0; chunk < 2; ++chunk) {
+                        const uint32_t *col = (const uint32_t *)slot + RGX_BUFFER_SIZE * 64 + chunk * (24 * 64) + lane;
+                        const float up = __builtin_nontemporal_load((const float *)slot + RGX_BUFFER_SIZE * 64 + 2 * 24 * 64 + chunk * 64 + lane);
+                        const f3 gs = g * up; // the chunk's power of two goes into dL/dC once instead of into 48 sums
+                        float v[48];
+#pragma unroll
+                        for (int j = 0; j < 24; ++j) {
+                            const uint32_t w = __builtin_nontemporal_load(col + j * 64);
+                            const float2 two = __half22float2(*(const __half2 *)&w);
+                            v[2 * j] = two.x;
+                            v[2 * j + 1] = two.y;
+                        }
+#pragma unroll
+                        for (int i = 0; i < RGX_CHUNK_SIZE; ++i)
+                            PB[chunk * RGX_CHUNK_SIZE + i] = fmaf(gs.x, v[3 * i], fmaf(gs.y, v[3 * i + 1], gs.z * v[3 * i + 2]));
+                    }
+                }
                 RGX_SEC(cn, RGX_SEC_SUMS);
             };
             // (2) prefix: PA <- a_k, PB <- (T_k e_k - D_k) dt - a_k e_k   (so X_k = PB + PA * g.c_i);
@@ -2245,8 +2295,8 @@ template <bool STATS>
 __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchParams P) { march_bwd<false, false, STATS>(P); }
 template <bool STATS>
 __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay(const MarchParams P) { march_bwd<true, false, STATS>(P); }
-template <bool STATS>
-__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay_sums(const MarchParams P) { march_bwd<true, true, STATS>(P); }
+template <bool STATS, bool HALF = false>
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay_sums(const MarchParams P) { march_bwd<true, true, STATS, HALF>(P); }
 
 // Test hook for the cooperative collect: per pixel a segment [tlo, thi] (thi < tlo = pixel idle);
 // writes each ray's hit count (negated when cut at cap) and the INPUT indices of its hits.
@@ -2420,6 +2470,8 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     P.sum_pool = nullptr;
     P.sum_next = nullptr;
     P.sum_slots = 0;
+    P.sum_slot_words = RGX_SUM_SLOT_WORDS;
+    if (march->record_format != 0 && march->record_format != 1) return RGX_EINVAL;
     return RGX_OK;
 }
 
@@ -2439,11 +2491,12 @@ static int attach_records(MarchParams &P, void *records, size_t records_bytes)
     const size_t words = records_bytes / sizeof(uint32_t) / ntiles;
     if (((uintptr_t)records & 15u) || words < RGX_REC_MIN_TILE_WORDS) return RGX_EWORKSPACE;
     P.records = (uint32_t *)records;
+    P.sum_slot_words = P.m.record_format == 1 ? RGX_SUM_SLOT_WORDS_HALF : RGX_SUM_SLOT_WORDS;
     if (words >= RGX_REC_LIST_WORDS + RGX_SUM_SLOT_WORDS) {
         // room beyond the hit lists: RGX_REC_LIST_WORDS per tile, a 256-byte pool header, the sample-sum slots
         P.rec_tile_words = RGX_REC_LIST_WORDS;
         const size_t head = ntiles * (size_t)RGX_REC_LIST_WORDS * sizeof(uint32_t);
-        const size_t slots = (records_bytes - head - 256) / (RGX_SUM_SLOT_WORDS * sizeof(uint32_t));
+        const size_t slots = (records_bytes - head - 256) / ((size_t)P.sum_slot_words * sizeof(uint32_t));
         P.sum_next = (uint32_t *)((char *)records + head);
         P.sum_pool = (float4 *)((char *)records + head + 256);
         P.sum_slots = (int32_t)(slots > 0x7fffffff ? 0x7fffffff : slots);
@@ -2515,7 +2568,10 @@ static int march_forward_launch(const void *ws, const RgxCamera *cam, const RgxM
     void *span = rgx_span_begin(RGX_T_MARCH_FWD, (hipStream_t)stream);
     if (P.sum_pool || P.faults) hipLaunchKernelGGL(k_clear2, dim3(1), dim3(64), 0, (hipStream_t)stream, (float4 *)P.sum_next, (float4 *)P.faults);
     order_blocks(P, (hipStream_t)stream);
-    if (P.records) {
+    if (P.records && P.sum_pool && P.m.record_format == 1) {
+        if (counting) hipLaunchKernelGGL((k_march_fwd<true, false, true, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+        else hipLaunchKernelGGL((k_march_fwd<true, false, false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
+    } else if (P.records) {
         if (counting) hipLaunchKernelGGL((k_march_fwd<true, false, true>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
         else hipLaunchKernelGGL((k_march_fwd<true, false, false>), march_grid(P), dim3(64), 0, (hipStream_t)stream, P);
     } else {
@@ -2636,11 +2692,14 @@ static int march_backward_launch(const void *ws, const RgxCamera *cam, const Rgx
             hipLaunchKernelGGL(k_tile_order, dim3(8), dim3(256), 0, s, P);
             P.use_tile_order = 1;
         }
+        const bool half = P.m.record_format == 1;
         if (stats) {
-            if (P.sum_pool) hipLaunchKernelGGL(k_march_bwd_replay_sums<true>, march_grid(P), dim3(64), 0, s, P);
+            if (P.sum_pool && half) hipLaunchKernelGGL((k_march_bwd_replay_sums<true, true>), march_grid(P), dim3(64), 0, s, P);
+            else if (P.sum_pool) hipLaunchKernelGGL((k_march_bwd_replay_sums<true, false>), march_grid(P), dim3(64), 0, s, P);
             hipLaunchKernelGGL(k_march_bwd_replay<true>, march_grid(P), dim3(64), 0, s, P);
         } else {
-            if (P.sum_pool) hipLaunchKernelGGL(k_march_bwd_replay_sums<false>, march_grid(P), dim3(64), 0, s, P);
+            if (P.sum_pool && half) hipLaunchKernelGGL((k_march_bwd_replay_sums<false, true>), march_grid(P), dim3(64), 0, s, P);
+            else if (P.sum_pool) hipLaunchKernelGGL((k_march_bwd_replay_sums<false, false>), march_grid(P), dim3(64), 0, s, P);
             hipLaunchKernelGGL(k_march_bwd_replay<false>, march_grid(P), dim3(64), 0, s, P);
         }
         P.only_overflow = 1;
@@ -2759,6 +2818,14 @@ extern "C" int rgx_debug_section_cycles(unsigned long long *host_out, int reset)
     }
     return RGX_OK;
 }
+// The raw table: 2 x RGX_SEC_ROWS x 16 words (see g_section_cycles), for per-workgroup timelines.
+extern "C" int rgx_debug_section_rows(unsigned *host_out)
+{
+    if (!host_out) return RGX_EINVAL;
+    RGX_HIP(hipDeviceSynchronize());
+    RGX_HIP(hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_section_cycles), sizeof(unsigned) * 2 * RGX_SEC_ROWS * 16));
+    return RGX_OK;
+}
 #endif
 
 // Test hook: counts the pairs for which the plain division or the plain square root differs in any
@@ -2785,33 +2852,68 @@ extern "C" int rgx_check_plain_arith(const float *a, const float *b, int64_t n, 
     return RGX_OK;
 }
 
-// Measurement hook: independent fp32 multiply-adds and nothing else (16 chains per lane, so that no
-// instruction waits for the one before), for the VALU issue rate of the card.
+// Measurement hook: one instruction repeated, sixteen independent registers per lane so that none waits for the one
+// before, for the rate at which the card issues that class of VALU instruction (asm volatile: the compiler may
+// neither fold nor reorder them).
+#define RGX_PROBE_REP16(S) S(0) S(1) S(2) S(3) S(4) S(5) S(6) S(7) S(8) S(9) S(10) S(11) S(12) S(13) S(14) S(15)
+template <int KIND>
 __global__ __launch_bounds__(256) void k_probe_valu(int iters, float seed, float *sink)
 {
     float a[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) a[i] = seed + (float)(threadIdx.x + i);
     const float m = 1.0f - seed * 1e-9f, c = seed * 1e-9f;
+    unsigned long long mask = __ballot(threadIdx.x & 1);
     for (int it = 0; it < iters; ++it) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) a[i] = fmaf(a[i], m, c);
+        for (int r = 0; r < 4; ++r) {
+#define RGX_P_FMA(i) asm volatile("v_fma_f32 %0, %0, %1, %2" : "+v"(a[i]) : "v"(m), "v"(c));
+#define RGX_P_ADD(i) asm volatile("v_add_f32 %0, %0, %1" : "+v"(a[i]) : "v"(c));
+#define RGX_P_MOV(i) asm volatile("v_mov_b32 %0, %1" : "=v"(a[i]) : "v"(m));
+#define RGX_P_AND(i) asm volatile("v_and_b32 %0, %0, %1" : "+v"(a[i]) : "v"(m));
+#define RGX_P_CMP(i) asm volatile("v_cmp_lt_f32 %0, %1, %2" : "=s"(mask) : "v"(a[i]), "v"(m));
+#define RGX_P_CND(i) asm volatile("v_cndmask_b32 %0, %0, %1, %2" : "+v"(a[i]) : "v"(m), "s"(mask));
+#define RGX_P_MAX(i) asm volatile("v_max_f32 %0, %0, %1" : "+v"(a[i]) : "v"(m));
+#define RGX_P_DPP(i) asm volatile("v_add_f32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf bound_ctrl:0" : "+v"(a[i]));
+#define RGX_P_SHL(i) asm volatile("v_lshlrev_b32 %0, 1, %0" : "+v"(a[i]));
+#define RGX_P_EXP(i) asm volatile("v_exp_f32 %0, %0" : "+v"(a[i]));
+            if constexpr (KIND == 0) { RGX_PROBE_REP16(RGX_P_FMA) }
+            else if constexpr (KIND == 1) { RGX_PROBE_REP16(RGX_P_ADD) }
+            else if constexpr (KIND == 2) { RGX_PROBE_REP16(RGX_P_MOV) }
+            else if constexpr (KIND == 3) { RGX_PROBE_REP16(RGX_P_AND) }
+            else if constexpr (KIND == 4) { RGX_PROBE_REP16(RGX_P_CMP) }
+            else if constexpr (KIND == 5) { RGX_PROBE_REP16(RGX_P_CND) }
+            else if constexpr (KIND == 6) { RGX_PROBE_REP16(RGX_P_MAX) }
+            else if constexpr (KIND == 7) { RGX_PROBE_REP16(RGX_P_DPP) }
+            else if constexpr (KIND == 8) { RGX_PROBE_REP16(RGX_P_SHL) }
+            else { RGX_PROBE_REP16(RGX_P_EXP) }
+        }
     }
     float t = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) t += a[i];
-    if (t == -1.2345f) *sink = t; // never for finite seeds: the sums stay positive
+    if (t == -1.2345f) *sink = t + (float)mask; // (practically never: keeps the registers live)
 }
 
-extern "C" int rgx_probe_valu_rate(int32_t waves, int32_t iters, float *sink, uint64_t *instructions, void *stream)
+extern "C" int rgx_probe_valu_rate(int32_t waves, int32_t iters, int32_t kind, float *sink, uint64_t *instructions, void *stream)
 {
-    if (waves <= 0 || iters <= 0 || !sink || !instructions) return RGX_EINVAL;
+    if (waves <= 0 || iters <= 0 || kind < 0 || kind > 9 || !sink || !instructions) return RGX_EINVAL;
     const DeviceScope on_device(sink);
-    const unsigned groups = (unsigned)((waves + 3) / 4);
-    hipLaunchKernelGGL(k_probe_valu, dim3(groups), dim3(256), 0, (hipStream_t)stream, (int)iters, 1.0f, sink);
-    *instructions = (uint64_t)groups * 4u * (uint64_t)iters * 64u;
+    const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+    hipStream_t s = (hipStream_t)stream;
+    switch (kind) {
+    case 0: hipLaunchKernelGGL(k_probe_valu<0>, grid, block, 0, s, (int)iters, 1.0f, sink); break;
+    case 1: hipLaunchKernelGGL(k_probe_valu<1>, grid, block, 0, s, (int)iters, 1.0f, sink); break;
+    case 2: hipLaunchKernelGGL(k_probe_valu<2>, grid, block, 0, s, (int)iters, 1.0f, sink); break;
+    case 3: hipLaunchKernelGGL(k_probe_valu<3>, grid, block, 0, s, (int)iters, 1.0f, sink); break;
+    case 4: hipLaunchKernelGGL(k_probe_valu<4>, grid, block, 0, s, (int)iters, 1.0f, sink); break;
+    case 5: hipLaunchKernelGGL(k_probe_valu<5>, grid, block, 0, s, (int)iters, 1.0f, sink); break;
+    case 6: hipLaunchKernelGGL(k_probe_valu<6>, grid, block, 0, s, (int)iters, 1.0f, sink); break;
+    case 7: hipLaunchKernelGGL(k_probe_valu<7>, grid, block, 0, s, (int)iters, 1.0f, sink); break;
+    case 8: hipLaunchKernelGGL(k_probe_valu<8>, grid, block, 0, s, (int)iters, 1.0f, sink); break;
+    default: hipLaunchKernelGGL(k_probe_valu<9>, grid, block, 0, s, (int)iters, 1.0f, sink); break;
+    }
+    *instructions = (uint64_t)grid.x * 4u * (uint64_t)iters * 64u;
     RGX_LAUNCH_CHECK();
     return RGX_OK;
 }

@@ -222,6 +222,7 @@ REC_FIRST_SLOTS = 12
 
 REC_LIST_WORDS = 16384        # the hit lists' share of a tile's record
 REC_SLOT_WORDS = 8192         # one slot of sample sums
+REC_SLOT_WORDS_HALF = 2048 + 2 * 24 * 64 + 2 * 64   # ... with half-precision colour sums (record_format 1)
 REC_MEMORY_SHARE = 0.4        # of the device's memory: the most a record may take by default
 
 
@@ -254,8 +255,12 @@ REC_POOL_STEP = 1 << 12       # ... rounded up to a multiple of this many slots 
 REC_POOL_HISTORY = 8
 
 
-def _usage_key(cam, device, n):
-    return (str(device), torch.cuda.current_stream(device).cuda_stream, int(n), cam.width, cam.height)
+def _usage_key(cam, device, n, record_format=0):
+    return (str(device), torch.cuda.current_stream(device).cuda_stream, int(n), cam.width, cam.height, int(record_format))
+
+
+def _slot_words(record_format):
+    return REC_SLOT_WORDS_HALF if record_format == 1 else REC_SLOT_WORDS
 
 
 def _pool_geometry(cam):
@@ -263,7 +268,7 @@ def _pool_geometry(cam):
     return ntiles, ntiles * REC_LIST_WORDS * 4        # tiles, bytes of the hit-list regions (the pool header follows)
 
 
-def new_records(cam, device, tile_words=REC_TILE_WORDS, budget_bytes=None, n=0):
+def new_records(cam, device, tile_words=REC_TILE_WORDS, budget_bytes=None, n=0, record_format=0):
     """Buffer for the record of one forward launch (see rgx_march_records_bytes), or None when no
     record fits the budget or the allocator.  The budget defaults to REC_MEMORY_SHARE of the device's
     memory and at most 80 % of what is free now.  With the default ``tile_words`` the pool of sample
@@ -276,13 +281,15 @@ def new_records(cam, device, tile_words=REC_TILE_WORDS, budget_bytes=None, n=0):
         free, total = torch.cuda.mem_get_info(device)
         budget_bytes = int(min(REC_MEMORY_SHARE * total, 0.8 * free))
     if tile_words == REC_TILE_WORDS:
-        key = _usage_key(cam, device, n)
+        key = _usage_key(cam, device, n, record_format)
         use = _rec_usage.get(key)
         if use is None:
             if len(_rec_usage) >= 64:
                 del _rec_usage[next(iter(_rec_usage))]
             use = _rec_usage[key] = dict(pinned=torch.zeros(1, dtype=torch.int32).pin_memory(), event=torch.cuda.Event(),
                                          pending=False, need=[], slots=0, allocated=0)
+        if use["pending"] and not use["need"]:
+            use["event"].synchronize()     # the second view of a key waits for the first view's count: once per key
         _read_record_use(use)
         ntiles, head = _pool_geometry(cam)
         have = use["slots"]
@@ -293,7 +300,7 @@ def new_records(cam, device, tile_words=REC_TILE_WORDS, budget_bytes=None, n=0):
         elif not have:
             have = REC_FIRST_SLOTS * ntiles
         have = max(min(have, 64 * ntiles), ntiles)     # (the library wants at least one slot per tile to keep sums at all)
-        nbytes = head + 256 + have * REC_SLOT_WORDS * 4
+        nbytes = max(head + 256 + have * _slot_words(record_format) * 4, ntiles * (REC_LIST_WORDS + REC_SLOT_WORDS) * 4)
         if nbytes <= budget_bytes:
             try:
                 rec = torch.empty(nbytes, dtype=torch.uint8, device=device)
@@ -316,12 +323,12 @@ def _read_record_use(use):
         use["need"] = (use["need"] + [int(use["pinned"][0])])[-REC_POOL_HISTORY:]
 
 
-def note_record_use(records, cam, device, n=0):
+def note_record_use(records, cam, device, n=0, record_format=0):
     """After a forward launch that wrote ``records``: queue a 4-byte copy of the pool's bump counter
     (the slots the launch asked for, also beyond the pool's end) to pinned host memory.  Nothing waits
     for it; the next ``new_records`` of this scene size and image shape on this stream reads it."""
     ntiles, head = _pool_geometry(cam)
-    use = _rec_usage.get(_usage_key(cam, device, n))
+    use = _rec_usage.get(_usage_key(cam, device, n, record_format))
     # (the library keeps sample sums only in a record with room for the hit lists and at least one slot per tile)
     if use is None or records is None or records.numel() // 4 // ntiles < REC_LIST_WORDS + REC_SLOT_WORDS:
         return
@@ -334,26 +341,26 @@ def note_record_use(records, cam, device, n=0):
     use["pending"] = True
 
 
-def record_use(cam, device, n=0):
+def record_use(cam, device, n=0, record_format=0):
     """(bytes allocated for the last record of this scene size and image shape on this stream, bytes the last
     launch read back asked for: hit-list regions + sample-sum slots), or None before the first launch has reported."""
-    use = _rec_usage.get(_usage_key(cam, device, n))
+    use = _rec_usage.get(_usage_key(cam, device, n, record_format))
     if use is None:
         return None
     _read_record_use(use)
     if not use["need"]:
         return None
     ntiles, head = _pool_geometry(cam)
-    return use["allocated"], head + 256 + use["need"][-1] * REC_SLOT_WORDS * 4
+    return use["allocated"], head + 256 + use["need"][-1] * _slot_words(record_format) * 4
 
 
 def march_forward(gas, cam, prims, dt_step, dynamic_sampling, max_prim_slice, white_background,
-                  t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None, ray_counts=False):
+                  t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None, ray_counts=False, record_format=0):
     """``ray_counts=True`` (test hook): also returns an (n_rays, 2) int32 tensor, per ray the slabs blended and
     the sum of their hit-list lengths."""
     n, dev = prims.shape[0], prims.device
     n_rays = cam.width * cam.height
-    m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), int(bool(white_background)), t_eps)
+    m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), int(bool(white_background)), t_eps, int(record_format))
     ws = _march_ws(n, n_rays, max_prim_slice, dev)
     ray_colors = torch.empty(n_rays, 3, dtype=torch.float32, device=dev)
     if ray_counts:
@@ -398,11 +405,11 @@ def sh_viewer(camera_center, positions, sh, sph_gauss_features, bandwidth_sharpn
 
 
 def march_backward(gas, cam, prims, ray_colors, dloss, dt_step, dynamic_sampling, max_prim_slice,
-                   white_background=True, t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None, out=None):
+                   white_background=True, t_eps=TRANSMITTANCE_EPSILON, stats=None, records=None, out=None, record_format=0):
     """``out``: five preallocated gradient tensors (density, rgb, position, scale, quaternion) to write into."""
     n, dev = prims.shape[0], prims.device
     n_rays = cam.width * cam.height
-    m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), int(bool(white_background)), t_eps)
+    m = L.RgxMarch(dt_step, int(bool(dynamic_sampling)), int(max_prim_slice), int(bool(white_background)), t_eps, int(record_format))
     ws = _march_ws(n, n_rays, max_prim_slice, dev)
     ddens, drgb, dpos, dscale, dquat = out if out is not None else (
         torch.empty(n, dtype=torch.float32, device=dev), torch.empty(n, 3, dtype=torch.float32, device=dev),

@@ -85,6 +85,9 @@ class RenderOptixSettings:
         self.stats = None   # optional optix_utils.new_stats() block
         self.record_hits = True   # forward records its hit lists for the backward to replay
         self.rec_tile_words = u_ox.REC_TILE_WORDS   # record size per 8x8 pixel tile, 32-bit words
+        # True: the record keeps the per-sample colour sums in half precision with a power-of-two scale per ray and
+        # 16 samples (two thirds of the record's bytes; gradients within about 1e-4 of those of the float record)
+        self.rec_half_sums = False
         # True: ``gas`` was built from these very positions, scales, quaternions and densities (an earlier
         # view of the same accumulation window) -- the forward then skips the rebuild
         self.gas_is_current = False
@@ -128,12 +131,14 @@ class RenderOptixFunction(torch.autograd.Function):
                           settings.num_sph_gauss, order_sh)
         prims = u_ox.pack_prims(gas, cam, positions, scales, normalized_quaternions, densities, rgb)
         # when a backward will follow, the forward leaves a record of its hit lists for it to replay
-        records = (u_ox.new_records(cam, dev, settings.rec_tile_words, n=n)
+        fmt = 1 if settings.rec_half_sums else 0
+        records = (u_ox.new_records(cam, dev, settings.rec_tile_words, n=n, record_format=fmt)
                    if (any(ctx.needs_input_grad[:8]) and settings.record_hits) else None)
         ray_colors = u_ox.march_forward(gas, cam, prims, settings.dt_step, settings.dynamic_sampling,
                                         settings.max_prim_slice, settings.white_background, settings.t_eps,
-                                        settings.stats, records)
-        u_ox.note_record_use(records, cam, dev, n)
+                                        settings.stats, records, record_format=fmt)
+        u_ox.note_record_use(records, cam, dev, n, fmt)
+        ctx.record_format = fmt
         ctx.records = records
         ctx.settings = settings
         ctx.cam = cam
@@ -153,7 +158,7 @@ class RenderOptixFunction(torch.autograd.Function):
             densities_grad, rgb_grad, positions_grad, scales_grad, quaternions_grad = u_ox.march_backward(
                 ctx.gas, ctx.cam, ctx.prims, ray_colors, dloss_dray_colors, settings.dt_step,
                 settings.dynamic_sampling, settings.max_prim_slice, settings.white_background, settings.t_eps,
-                settings.stats, ctx.records)
+                settings.stats, ctx.records, record_format=ctx.record_format)
             ctx.records = None
             ws = u_ox._scratch.get(("march", str(positions.device), torch.cuda.current_stream(positions.device).cuda_stream))
             if ws is not None:

@@ -20,7 +20,7 @@ def cos_rel(a, b):
 
 
 def gpu_render(scene_np, cam, cfg, white=True, supersampling=(1, 1), want_grad=None, stats=True, record_hits=True,
-               rec_tile_words=None):
+               rec_tile_words=None, half_sums=False):
     """Runs RenderOptixFunction (and its backward when ``want_grad`` = dL/dimage is given).
     ``record_hits``: the backward replays the forward's hit-list record (the default) or searches
     the tree again; ``rec_tile_words`` sizes the record per tile."""
@@ -38,6 +38,7 @@ def gpu_render(scene_np, cam, cfg, white=True, supersampling=(1, 1), want_grad=N
                                 num_sph_gauss=g, white_background=white, supersampling=supersampling,
                                 t_eps=cfg.get("t_eps", 1e-3))
     settings.record_hits = record_hits
+    settings.rec_half_sums = half_sums
     if rec_tile_words is not None:
         settings.rec_tile_words = rec_tile_words
     if stats:

@@ -596,3 +596,48 @@ def test_training_stress_1M_1024x1024_windows_with_reorder_and_rebuild(gx, orc):
     for k in PARAMS:
         cos, rel = gx.cos_rel(b["grads"][k], a["grads"][k][order_np])
         assert cos >= 1 - 1e-6 and rel <= 1e-4, (k, cos, rel)
+
+
+def test_half_precision_colour_sums_in_the_record(gx, orc, big):
+    """settings.rec_half_sums: the record keeps the per-sample colour sums in half precision with a power-of-two
+    scale per ray and 16 samples (record_format 1 of the C ABI).  The image does not depend on the record; the
+    gradients must stay within the gates of the oracle's at the benchmark's size and close to the float record's.
+    With densities of 1e6, where the sums leave binary16's range, the scale keeps them finite and 11 bits exact --
+    what plain half precision could not do -- but every sample is then one opaque Gaussian's, g.c_i - e_k cancels
+    to the sums' last bits, and the gradients are only good to a few per cent: why the format is an option."""
+    sc, cam, cfg = big
+    ids = np.linspace(0, W * H - 1, 384).astype(np.int64)
+    img, st, ctx = orc.render_forward(sc, cam, cfg["dt_step"], cfg["dynamic_sampling"], cfg["max_prim_slice"], ray_ids=ids, cull=True)
+    stable = gx.cutoff_stable_rays(orc, ctx, img, ids)
+    dloss = np.zeros((W * H, 3), np.float32)
+    dloss[ids[stable]] = np.random.default_rng(71).normal(size=(int(stable.sum()), 3)).astype(np.float32)
+    og, _ = orc.render_backward(sc, ctx, img, dloss)
+    _step("1 M Gaussians, 800x800: float and half-precision colour sums, twice each (the second view's pool is sized from the first)")
+    outs = {}
+    for half in (False, True):
+        for _ in range(2):
+            outs[half] = gx.gpu_render(sc, cam, cfg, want_grad=dloss, stats=True, half_sums=half)
+        assert outs[half]["stats_bwd"]["nodes_visited"] == 0 and outs[half]["stats_bwd"]["replay_lost"] == 0
+    assert np.array_equal(outs[True]["image"], outs[False]["image"])
+    for k in PARAMS:
+        cos, rel = gx.cos_rel(outs[True]["grads"][k], og[k])
+        cos2, rel2 = gx.cos_rel(outs[True]["grads"][k], outs[False]["grads"][k])
+        print(f"half sums, {k}: against the oracle 1 - cos {1 - cos:.2e}, rel {rel:.2e}; against the float record rel {rel2:.2e}", flush=True)
+        assert cos >= COS_MIN and rel <= REL_MAX, (k, cos, rel)
+        assert rel2 <= 3e-4, (k, rel2)
+    # densities and colours far beyond binary16's range
+    small = scenes.scene_to_numpy(scenes.make_scene(0, n=3000, seed=72))
+    small = {k: small[k] for k in PARAMS}
+    small["densities"] = (small["densities"] * 1e6).astype(np.float32)
+    small["color_features"] = (small["color_features"] * 30.0).astype(np.float32)
+    cam0, cfg0 = scenes.make_camera(0, 0, width=96, height=96), scenes.CONFIGS[0]
+    g = np.random.default_rng(73).normal(size=(96 * 96, 3)).astype(np.float32)
+    _step("densities of 1e6: float and half-precision colour sums")
+    a = gx.gpu_render(small, cam0, cfg0, want_grad=g, half_sums=False)
+    b = gx.gpu_render(small, cam0, cfg0, want_grad=g, half_sums=True)
+    assert np.array_equal(a["image"], b["image"])
+    for k in PARAMS:
+        assert np.isfinite(b["grads"][k]).all(), k
+        cos, rel = gx.cos_rel(b["grads"][k], a["grads"][k])
+        print(f"densities of 1e6, {k}: half against float record rel {rel:.2e}", flush=True)
+        assert cos >= 0.995 and rel <= 0.1, (k, cos, rel)      # measured: 3e-2 at worst (positions)

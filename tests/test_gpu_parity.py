@@ -671,7 +671,7 @@ def test_direct_ctypes_binding_matches_the_python_mirror(gx, c0):
 
     class RgxMarch(C.Structure):
         _fields_ = [("dt_step", C.c_float), ("dynamic_sampling", C.c_int32), ("max_prim_slice", C.c_int32),
-                    ("white_background", C.c_int32), ("t_eps", C.c_float)]
+                    ("white_background", C.c_int32), ("t_eps", C.c_float), ("record_format", C.c_int32)]
 
     def p(t):
         return C.c_void_p(t.data_ptr())

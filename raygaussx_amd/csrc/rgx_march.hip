@@ -2296,7 +2296,10 @@ __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd(const MarchPara
 template <bool STATS>
 __global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay(const MarchParams P) { march_bwd<true, false, STATS>(P); }
 template <bool STATS, bool HALF = false>
-__global__ __launch_bounds__(64) RGX_WAVES_ATTR void k_march_bwd_replay_sums(const MarchParams P) { march_bwd<true, true, STATS, HALF>(P); }
+#ifndef RGX_WAVES_ATTR_SUMS
+#define RGX_WAVES_ATTR_SUMS RGX_WAVES_ATTR
+#endif
+__global__ __launch_bounds__(64) RGX_WAVES_ATTR_SUMS void k_march_bwd_replay_sums(const MarchParams P) { march_bwd<true, true, STATS, HALF>(P); }
 
 // Test hook for the cooperative collect: per pixel a segment [tlo, thi] (thi < tlo = pixel idle);
 // writes each ray's hit count (negated when cut at cap) and the INPUT indices of its hits.

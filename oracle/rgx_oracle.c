@@ -41,6 +41,12 @@
  *                       its dynamic_sampling branch: autograd is fed the forward's
  *                       (pinned) slab sequence, so a backward that stepped
  *                       differently would miss its gradients
+ *   orc_march_backward_in_cut / orc_set_backward_mask_form (probes of the backward's
+ *                       cut-off decisions): the count against a float64 count over the same
+ *                       slabs on every ray with no sample within rounding of a cut-off; the
+ *                       forward's form of the decision leaves every Gaussian alone that no
+ *                       disagreeing ray touches
+ *   orc_cull_build      brute force (same candidates, bit for bit)
  *   orc_march_gui       float64 quadrature of int t sigma exp(-tau) dt for one Gaussian,
  *                       depth / (1 - T) inside the scene box, known quantisation values
  *   orc_morton_codes    naive per-bit loop

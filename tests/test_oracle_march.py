@@ -477,3 +477,71 @@ def test_step_scale_probe_is_exact_at_one_and_moves_the_adaptive_march(orc):
         orc.set_step_scale(1.0)
     img_e, _, _ = orc.render_forward(sc, cam, cfg["dt_step"], False, cfg["max_prim_slice"])
     assert np.array_equal(img_d, img_e)
+
+
+def test_cutoff_probes_of_the_backward(orc):
+    """orc_march_backward_in_cut / orc_set_backward_mask_form: the per-ray count of samples the backward's
+    gradient loop takes as inside a cut-off equals a float64 count over the same slabs on every ray without a
+    sample within rounding of a cut-off; the count of samples on which the forward's and the backward's
+    arrangements of the power disagree is zero on almost every ray, and never more than the float64 count's
+    near-edge samples; deciding by the forward's arrangement changes the gradients of no Gaussian that no
+    disagreeing ray touches, and leaves everything alone when no ray disagrees."""
+    sc = scenes.scene_to_numpy(scenes.make_scene(0, n=500, sh_degree=0, seed=41))
+    sc["scales"] = sc["scales"] * 2.0
+    sc["densities"] = sc["densities"] * 0.25 + 0.12          # faint: no ray saturates, every blended sample counts
+    cam = scenes.make_camera(0, 0, width=20, height=20)
+    img, st, ctx = orc.render_forward(sc, cam, 0.0025, False, 500)
+    args = (ctx["cs"], ctx["ms"], ctx["bmin"], ctx["bmax"], ctx["prims"])
+    counts = orc.march_backward_in_cut(*args, img)
+    assert counts.shape == (400, 2) and counts[:, 0].sum() > 20000
+    eye = cam.camera_center.double().numpy()
+    dirs = f64ref.ray_dirs_pinhole(cam)
+    R = f64ref.rot_from_quat(torch.tensor(sc["quaternions"].astype(np.float64))).numpy()
+    pos, scale = sc["positions"].astype(np.float64), sc["scales"].astype(np.float64)
+    kk = 2.0 * np.log(sc["densities"].astype(np.float64) / 0.1)
+    want, near = np.zeros(400, np.int64), np.zeros(400, np.int64)
+    touched = [set() for _ in range(400)]
+    for r in range(400):
+        slabs, _ = orc.march_trace(*args, r)
+        for tb, dt, tlo, thi, ids in slabs:
+            if not len(ids):
+                continue
+            touched[r].update(int(i) for i in ids)
+            t = tb + dt * (np.arange(32) + 0.5)
+            x = eye[None] + t[:, None] * dirs[r][None]
+            loc = np.einsum("hji,hsj->hsi", R[ids], x[None] - pos[ids][:, None]) / scale[ids][:, None]
+            power = (loc ** 2).sum(-1)
+            want[r] += int((power < kk[ids][:, None]).sum())
+            near[r] += int((np.abs(power / kk[ids][:, None] - 1.0) < 2e-4).sum())     # one ulp of t moves a thin Gaussian's power by 1e-4
+    clear = near == 0
+    assert clear.mean() > 0.8
+    assert np.array_equal(counts[clear, 0], want[clear])                 # the count itself, against float64
+    assert np.all(np.abs(counts[:, 0] - want) <= near)
+    assert np.all(counts[:, 1] <= near) and (counts[:, 1] == 0).mean() > 0.97
+    # the two forms of the decision
+    rng = np.random.default_rng(42)
+    dloss = rng.normal(size=img.shape).astype(np.float32)
+    g0, _ = orc.march_backward(*args, img, dloss)
+    orc.set_backward_mask_form(1)
+    try:
+        g1, _ = orc.march_backward(*args, img, dloss)
+        again = orc.march_backward_in_cut(*args, img)
+    finally:
+        orc.set_backward_mask_form(0)
+    assert np.array_equal(again, counts)                                 # the probe reports both forms whichever decides
+    disagreeing = np.nonzero(counts[:, 1] > 0)[0]
+    suspects = set().union(*[touched[r] for r in disagreeing]) if len(disagreeing) else set()
+    same = np.ones(500, bool)
+    same[list(suspects)] = False
+    for k in g0:
+        assert np.array_equal(g0[k][same], g1[k][same]), k
+    quiet = dloss.copy()
+    quiet[disagreeing] = 0.0
+    h0, _ = orc.march_backward(*args, img, quiet)
+    orc.set_backward_mask_form(1)
+    try:
+        h1, _ = orc.march_backward(*args, img, quiet)
+    finally:
+        orc.set_backward_mask_form(0)
+    for k in h0:
+        assert np.array_equal(h0[k], h1[k]), k                          # without the disagreeing rays: the same backward, bit for bit

@@ -322,6 +322,8 @@ def side_kernels(dev, reps):
 SECTION_NAMES = ("sweep", "filter", "shade_or_gradient_trips", "record_lists", "blend_or_prefix", "sample_sums_io",
                  "tile_setup", "iteration_top", "iteration_end", "epilogue", "walk_and_parse", "flush_gradients")
 SECTION_KERNELS = ("k_march_fwd<record>", "k_march_fwd<plain>", "k_march_bwd_replay_sums", "k_march_bwd_replay", "k_march_bwd")
+# the replaying backward sweeps and filters nothing: it files the parts of its walk under those sections
+REPLAY_SECTION_NAMES = {"sweep": "parse_items", "filter": "count_hits_and_set_windows_up", "record_lists": "first_words_of_the_lists"}
 
 
 def read_sections(reset=False):
@@ -339,7 +341,8 @@ def read_sections(reset=False):
         total = sum(row[:nsec])
         if row[nsec] and total:
             out[kernel] = dict(waves=row[nsec], cycles_per_wave=round(total / row[nsec]),
-                               shares={name: round(c / total, 4) for name, c in zip(SECTION_NAMES, row[:nsec]) if c})
+                               shares={(REPLAY_SECTION_NAMES.get(name, name) if "replay" in kernel else name): round(c / total, 4)
+                                       for name, c in zip(SECTION_NAMES, row[:nsec]) if c})
     return out
 
 

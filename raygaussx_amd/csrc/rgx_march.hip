@@ -92,6 +92,7 @@ struct MarchParams {
 #define RGX_NSEC 12
 enum { RGX_SEC_SWEEP = 0, RGX_SEC_FILTER = 1, RGX_SEC_SHADE = 2, RGX_SEC_LISTS = 3, RGX_SEC_BLEND = 4, RGX_SEC_SUMS = 5,
        RGX_SEC_SETUP = 6, RGX_SEC_TOP = 7, RGX_SEC_END = 8, RGX_SEC_EPILOGUE = 9, RGX_SEC_WALK = 10, RGX_SEC_FLUSH = 11 };
+enum { RGX_SEC_PARSE = RGX_SEC_SWEEP, RGX_SEC_COUNT = RGX_SEC_FILTER, RGX_SEC_PRETRIP = RGX_SEC_LISTS }; // the replaying backward's names for sections it has no other use for
 enum { RGX_SECK_FWD_RECORD = 0, RGX_SECK_FWD_PLAIN = 1, RGX_SECK_BWD_SUMS = 2, RGX_SECK_BWD_LISTS = 3, RGX_SECK_BWD_TREE = 4, RGX_NSECK = 5 };
 #define RGX_SEC_ROWS 65536 // workgroups per launch the table has rows for (a 1920x1080 launch has 33 024)
 // [forward / backward][workgroup][section]; word RGX_NSEC of a row counts the waves that used it, the next word names their
@@ -1241,6 +1242,47 @@ __device__ __forceinline__ void sums_to_gradients(const Prim *pr, const float *s
 // column of RGX_NSUM per table slot): a row's share is added there with LDS atomics, and the
 // gradients go to memory once per window instead of once per row, slab and Gaussian.
 #define RGX_SLOT_TOUCHED 0x80000000u
+// The record as the replay reads it: the tile's region in memory, of which the words
+// [at, at + RGX_STAGE_WORDS) are also held in LDS once stage() has fetched them.  An iteration's items are
+// read word by word, each read depending on the last (a head gives a size gives the next head), and from
+// memory every link of that chain is a round trip; staged, the chain costs one.  Words outside the staged
+// range are read from memory as before.
+#define RGX_STAGE_WORDS 512
+template <bool STAGED>
+struct RecordView {
+    const uint32_t *reg; // the tile's region
+    uint32_t *lds;       // [RGX_STAGE_WORDS] (STAGED)
+    int at;              // first staged word (wave-uniform)
+    int used;            // words the forward wrote
+    __device__ __forceinline__ uint32_t word(int i) const
+    {
+        if constexpr (STAGED) {
+            const unsigned o = (unsigned)(i - at);
+            return o < (unsigned)RGX_STAGE_WORDS ? lds[o] : reg[i];
+        } else {
+            return reg[i];
+        }
+    }
+    __device__ __forceinline__ uint32_t uni(int i) const { return (uint32_t)__builtin_amdgcn_readfirstlane((int)word(i)); }
+    __device__ __forceinline__ uint32_t byte(int i, int b) const { return (word(i + (b >> 2)) >> ((b & 3) * 8)) & 0xffu; } // byte b after word i
+    __device__ __forceinline__ void stage(int from)
+    {
+        if constexpr (STAGED) {
+            uint32_t v[RGX_STAGE_WORDS / 64];
+#pragma unroll
+            for (int k = 0; k < RGX_STAGE_WORDS / 64; ++k) {
+                const int i = from + k * 64 + (int)threadIdx.x;
+                v[k] = i < used ? reg[i] : 0u;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int k = 0; k < RGX_STAGE_WORDS / 64; ++k) lds[k * 64 + threadIdx.x] = v[k];
+            at = from;
+            __syncthreads();
+        }
+    }
+};
+
 struct ReplayLds {
     float *acc;        // [RGX_NSUM][RGX_CCAP], component-major so that different slots fall in different banks
     uint32_t *pid;     // [RGX_CCAP]: the window's Gaussians by slot; top bit: the slot has something in acc
@@ -1275,14 +1317,14 @@ __device__ __forceinline__ void replay_flush(const MarchParams &P, const ReplayL
 }
 
 // Makes the WINDOW item at `at` the current window (sums of the previous one go to memory first).
-template <typename Cn>
-__device__ __forceinline__ void replay_window(const MarchParams &P, const ReplayLds &RL, const uint32_t *reg, int at, int &win_at, Cn &cn)
+template <typename Cn, typename Rv>
+__device__ __forceinline__ void replay_window(const MarchParams &P, const ReplayLds &RL, const Rv &rv, int at, int &win_at, Cn &cn)
 {
     if (at == win_at) return;
     replay_flush(P, RL, cn);
-    const int C = (int)(uni_u32(reg[at]) & 0xffffu);
+    const int C = (int)(rv.uni(at) & 0xffffu);
     for (int i = threadIdx.x; i < C && i < RGX_CCAP; i += 64) {
-        const uint32_t pid = min(reg[at + 4 + i], (uint32_t)(P.n - 1));
+        const uint32_t pid = min(rv.word(at + 4 + i), (uint32_t)(P.n - 1));
         RL.pid[i] = pid;
         const Prim *pr = P.prims + pid;
         f3 U, V, W;
@@ -1300,27 +1342,27 @@ __device__ __forceinline__ void replay_window(const MarchParams &P, const Replay
 // step); WALK 0 / 1: as shade_lanes over one half's entries; WALK_LANES_ALL: every ray walks all
 // its hits; WALK_NONE: no walk.  COUNT adds the lane's hits to p0.  Returns the item's size.
 enum { WALK_LANES_ALL = 2, WALK_ROWS_ALL = 3, WALK_NONE = 4 };
-template <bool COUNT, int WALK, typename Body>
-__device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLds &RL, const uint32_t *it, bool run, int &p0, Body body)
+template <bool COUNT, int WALK, typename Body, typename Cn, typename Rv>
+__device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLds &RL, const Rv &rv, int it, bool run, int &p0, Body body, Cn &cn)
 {
     const int lane = threadIdx.x, row = lane >> 4;
-    const int nw = (int)(uni_u32(it[0]) & 0xffu);
-    const int l0 = (int)uni_u32(it[1]), l1 = (int)uni_u32(it[2]), l2 = (int)uni_u32(it[3]), l3 = (int)uni_u32(it[4]);
+    const int nw = (int)(rv.uni(it) & 0xffu);
+    const int l0 = (int)rv.uni(it + 1), l1 = (int)rv.uni(it + 2), l2 = (int)rv.uni(it + 3), l3 = (int)rv.uni(it + 4);
     const int q0 = (l0 + 3) >> 2, q1 = (l1 + 3) >> 2, q2 = (l2 + 3) >> 2, q3 = (l3 + 3) >> 2;
     const int len = row == 0 ? l0 : row == 1 ? l1 : row == 2 ? l2 : l3;
-    const uint8_t *slots = (const uint8_t *)(it + 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0));
-    const uint32_t *masks = it + 8 + q0 + q1 + q2 + q3 + lane; // word w of this lane: masks[w * 64]
+    const int slots_at = it + 8 + (row > 0 ? q0 : 0) + (row > 1 ? q1 : 0) + (row > 2 ? q2 : 0); // the row's slot bytes start at this word
+    const int masks_at = it + 8 + q0 + q1 + q2 + q3 + lane;                                      // word w of this lane: masks_at + w * 64
     (void)RL.rowlist;
     if constexpr (WALK == WALK_NONE) {
         const int nwr = run ? min((len + 31) >> 5, nw) : 0;
         if (COUNT)
-            for (int w = 0; w < nwr; ++w) p0 += __popc(masks[w * 64]);
+            for (int w = 0; w < nwr; ++w) p0 += __popc(rv.word(masks_at + w * 64));
     } else if constexpr (WALK != WALK_ROWS_ALL) {
         const int nwr = run ? min((len + 31) >> 5, nw) : 0; // words of this lane's row; later words are not its own
-        const uint32_t *half = it + 8 + q0 + q1 + q2 + q3 + nw * 64 + ((WALK & 1) * 4 + row) * nw;
-        auto word = [&](int w) { return WALK == WALK_LANES_ALL ? masks[w * 64] : masks[w * 64] & half[w]; };
+        const int half_at = it + 8 + q0 + q1 + q2 + q3 + nw * 64 + ((WALK & 1) * 4 + row) * nw;
+        auto word = [&](int w) { return WALK == WALK_LANES_ALL ? rv.word(masks_at + w * 64) : rv.word(masks_at + w * 64) & rv.word(half_at + w); };
         if (COUNT)
-            for (int w = 0; w < nwr; ++w) p0 += __popc(masks[w * 64]);
+            for (int w = 0; w < nwr; ++w) p0 += __popc(rv.word(masks_at + w * 64));
         int w = 0;
         uint32_t bits = nwr > 0 ? word(0) : 0u;
         for (;;) {
@@ -1329,7 +1371,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
             if (!__any(has)) break;
             int slot = 0;
             if (has) {
-                slot = min((int)slots[w * 32 + __builtin_ctz(bits)], RGX_CCAP - 1);
+                slot = min((int)rv.byte(slots_at, w * 32 + __builtin_ctz(bits)), RGX_CCAP - 1);
                 bits &= bits - 1u;
             }
             const int32_t pid = (int32_t)(RL.pid[slot] & ~RGX_SLOT_TOUCHED);
@@ -1337,13 +1379,14 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
         }
     } else {
         const int maxlen = min(max(max(l0, l1), max(l2, l3)), nw * 32);
+        RGX_SEC(cn, RGX_SEC_WALK);
         // the rows' slot lists go to LDS first: every trip starts by looking its slot up, and from memory that
         // look-up is a round trip at the head of the trip's chain of dependent loads
+        const uint8_t *slots = RL.rowlist + row * RGX_CCAP;
         {
             uint32_t *dst = (uint32_t *)(RL.rowlist + row * RGX_CCAP);
-            for (int i = lane & 15; i < min((len + 3) >> 2, RGX_CCAP / 4); i += 16) dst[i] = ((const uint32_t *)slots)[i];
+            for (int i = lane & 15; i < min((len + 3) >> 2, RGX_CCAP / 4); i += 16) dst[i] = rv.word(slots_at + i);
             __syncthreads();
-            slots = RL.rowlist + row * RGX_CCAP;
         }
         static_assert(!COUNT, "the rows' walk counts nothing");
         (void)maxlen;
@@ -1353,7 +1396,7 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
         const int nwr = min((len + 31) >> 5, nw);
         auto lane_word = [&](int w) {
             const int left = len - w * 32;
-            return (run ? masks[w * 64] : 0u) & (left >= 32 ? ~0u : ((1u << left) - 1u));
+            return (run ? rv.word(masks_at + w * 64) : 0u) & (left >= 32 ? ~0u : ((1u << left) - 1u));
         };
         auto group_or = [](uint32_t m) {
             m |= (uint32_t)__builtin_amdgcn_update_dpp(0, (int)m, 0xB1, 0xf, 0xf, true);  // quad_perm [1,0,3,2]
@@ -1364,6 +1407,10 @@ __device__ __forceinline__ int replay_lists(const MarchParams &P, const ReplayLd
         int w = 0;
         uint32_t mword = nwr > 0 ? lane_word(0) : 0u;
         uint32_t bits = group_or(mword);
+#ifdef RGX_SECTION_CLOCKS
+        asm volatile("" :: "v"(bits)); // the first words have arrived: their wait belongs to the set-up, not to the first trip
+#endif
+        RGX_SEC(cn, RGX_SEC_PRETRIP);
         for (;;) {
             // (all lanes of a group hold the same bits and the same w: the DPP moves below run with the whole group active)
             while (__any(bits == 0u && w + 1 < nwr)) {
@@ -1561,17 +1608,18 @@ __device__ __forceinline__ bool slab_tables(const MarchParams &P, const TileLds 
 }
 
 // Size in words of the LISTS item at `it`.
-__device__ __forceinline__ int lists_size(const uint32_t *it)
+template <typename Rv>
+__device__ __forceinline__ int lists_size(const Rv &rv, int it)
 {
-    const int nw = (int)(uni_u32(it[0]) & 0xffu);
-    const int l0 = (int)uni_u32(it[1]), l1 = (int)uni_u32(it[2]), l2 = (int)uni_u32(it[3]), l3 = (int)uni_u32(it[4]);
+    const int nw = (int)(rv.uni(it) & 0xffu);
+    const int l0 = (int)rv.uni(it + 1), l1 = (int)rv.uni(it + 2), l2 = (int)rv.uni(it + 3), l3 = (int)rv.uni(it + 4);
     return 8 + ((l0 + 3) >> 2) + ((l1 + 3) >> 2) + ((l2 + 3) >> 2) + ((l3 + 3) >> 2) + nw * 72;
 }
 
 // Walks the record stream of one tile for the backward.
+template <bool STAGED>
 struct Replayer {
-    const uint32_t *reg; // the tile's region
-    int used;            // words the forward wrote
+    RecordView<STAGED> rv; // the tile's region
     int at;              // next item
     int win_at;          // the WINDOW item whose Gaussians sit in RL.pid (-1: none yet)
     bool lost;           // the stream did not hold the items an iteration expects (the caller stops)
@@ -1584,19 +1632,20 @@ struct Replayer {
     __device__ __forceinline__ bool slab(const MarchParams &P, const RayState &R, bool need, int &p0, float &found,
                                          float &searched_to, Cn &cn, BodyA body_a, Mid mid, BodyB body_b)
     {
-        const int start = at;
+        const int start = at, used = rv.used;
+        rv.stage(start);
         int end = at; // the iteration's TRAIL item
         for (;;) {
             if (end + 4 > used) break;
-            const uint32_t head = uni_u32(reg[end]);
+            const uint32_t head = rv.uni(end);
             int size;
             if ((head & 0xff000000u) == RGX_REC_WINDOW) size = 4 + (((int)(head & 0xffffu) + 3) & ~3);
-            else if ((head & 0xff000000u) == RGX_REC_LISTS && end + 8 <= used) size = lists_size(reg + end);
+            else if ((head & 0xff000000u) == RGX_REC_LISTS && end + 8 <= used) size = lists_size(rv, end);
             else break;
             if (end + size > used) break;
             end += size;
         }
-        const uint32_t tr = end + 4 <= used ? uni_u32(reg[end]) : 0u;
+        const uint32_t tr = end + 4 <= used ? rv.uni(end) : 0u;
         const bool any_search = tr & 1u;
         if ((tr & 0xff000000u) != RGX_REC_TRAIL || end + 4 + (any_search ? 64 : 0) > used) {
             lost = true;
@@ -1604,19 +1653,21 @@ struct Replayer {
             return false;
         }
         int dummy = 0;
+        RGX_SEC(cn, RGX_SEC_PARSE);
         if constexpr (SUMS) {
             auto none = [](const auto &, bool, bool, auto) {};
             for (int a = start; a < end;) {
-                const uint32_t head = uni_u32(reg[a]);
+                const uint32_t head = rv.uni(a);
                 if ((head & 0xff000000u) == RGX_REC_WINDOW) {
-                    replay_window(P, RL, reg, a, win_at, cn); // later iterations of the window carry no WINDOW item
+                    replay_window(P, RL, rv, a, win_at, cn); // later iterations of the window carry no WINDOW item
                     a += 4 + (((int)(head & 0xffffu) + 3) & ~3);
                 } else {
-                    a += replay_lists<true, WALK_NONE>(P, RL, reg + a, need, p0, none);
+                    a += replay_lists<true, WALK_NONE>(P, RL, rv, a, need, p0, none, cn);
                 }
             }
+            RGX_SEC(cn, RGX_SEC_COUNT);
             if (__any(need && p0 > 0)) {
-                const uint32_t slot1 = uni_u32(reg[end + 2]);
+                const uint32_t slot1 = rv.uni(end + 2);
                 if (slot1 == 0u || slot1 > (uint32_t)P.sum_slots) {
                     lost = true;
                     mid(false);
@@ -1626,29 +1677,29 @@ struct Replayer {
             }
         } else {
             for (int a = start; a < end;) {
-                const uint32_t head = uni_u32(reg[a]);
+                const uint32_t head = rv.uni(a);
                 if ((head & 0xff000000u) == RGX_REC_WINDOW) {
-                    replay_window(P, RL, reg, a, win_at, cn);
+                    replay_window(P, RL, rv, a, win_at, cn);
                     a += 4 + (((int)(head & 0xffffu) + 3) & ~3);
                 } else {
-                    replay_lists<true, 0>(P, RL, reg + a, need, p0, body_a);
-                    a += replay_lists<false, 1>(P, RL, reg + a, need, dummy, body_a);
+                    replay_lists<true, 0>(P, RL, rv, a, need, p0, body_a, cn);
+                    a += replay_lists<false, 1>(P, RL, rv, a, need, dummy, body_a, cn);
                 }
             }
         }
-        const float cover = __uint_as_float(uni_u32(reg[end + 1]));
-        found = any_search ? __uint_as_float(reg[end + 4 + threadIdx.x]) : -1.0f;
+        const float cover = __uint_as_float(rv.uni(end + 1));
+        found = any_search ? __uint_as_float(rv.word(end + 4 + (int)threadIdx.x)) : -1.0f;
         searched_to = fminf(R.texit, cover);
         at = end + 4 + (any_search ? 64 : 0);
         const bool run = mid(false);
         if (__any(run)) {
             for (int b = start; b < end;) {
-                const uint32_t head = uni_u32(reg[b]);
+                const uint32_t head = rv.uni(b);
                 if ((head & 0xff000000u) == RGX_REC_WINDOW) {
-                    replay_window(P, RL, reg, b, win_at, cn);
+                    replay_window(P, RL, rv, b, win_at, cn);
                     b += 4 + (((int)(head & 0xffffu) + 3) & ~3);
                 } else {
-                    b += replay_lists<false, WALK_ROWS_ALL>(P, RL, reg + b, run, dummy, body_b);
+                    b += replay_lists<false, WALK_ROWS_ALL>(P, RL, rv, b, run, dummy, body_b, cn);
                 }
             }
         }
@@ -1917,6 +1968,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
     __shared__ uint32_t s_pid[REPLAY ? RGX_CCAP : 1];
     __shared__ float s_frame[REPLAY ? 9 * RGX_CCAP : 1];
     __shared__ __align__(4) uint8_t s_rowlist[REPLAY ? 4 * RGX_CCAP : 4];
+    __shared__ uint32_t s_stage[REPLAY && SUMS ? RGX_STAGE_WORDS : 1]; // (with it the kernel's LDS comes to the forward's 12 800 bytes)
     const ReplayLds RL = {s_acc, s_pid, s_frame, s_rowlist};
     if constexpr (REPLAY) {
         for (int i = lane; i < RGX_NSUM * RGX_CCAP; i += 64) s_acc[i] = 0.f;
@@ -2133,14 +2185,15 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
 
     RGX_SEC(cn, RGX_SEC_SETUP);
     if constexpr (REPLAY) {
-        Replayer rp = {reg, min((int)uni_u32(reg[1]), P.rec_tile_words), 4, -1, false, RL};
+        const int used = min((int)uni_u32(reg[1]), P.rec_tile_words);
+        Replayer<SUMS> rp = {RecordView<SUMS>{reg, s_stage, -(1 << 30), used}, 4, -1, false, RL};
         while (__any(R.active) && !rp.lost) {
             iteration([&](bool need, float, float, int &p0, bool &, float &found, float &searched_to, auto a, auto mid, auto b) {
                 return rp.template slab<SUMS>(P, R, need, p0, found, searched_to, cn, a, mid, b);
             });
         }
         replay_flush(P, RL, cn);
-        if ((rp.lost || rp.at != rp.used) && lane == 0) {
+        if ((rp.lost || rp.at != rp.rv.used) && lane == 0) {
             cn.replay_lost = 1;
             if (P.faults) atomicAdd(&P.faults[0], 1u); // counted with or without a statistics block
         }

@@ -1071,6 +1071,9 @@ __device__ __forceinline__ void shade_lanes(const MarchParams &P, const TileLds 
 // the format safe for any density (plain binary16 overflows at 65504); the sums keep 11 bits relative to each
 // value down to 2^-14 of the chunk's largest.
 #define RGX_SUM_SLOT_WORDS_HALF (2048 + 2 * 24 * 64 + 2 * 64)
+#ifndef RGX_SUM_SLOT_BATCH
+#define RGX_SUM_SLOT_BATCH 2       // slots a tile takes from the pool at a time (the last batch's unused ones stay empty)
+#endif
 #define RGX_REC_COMPLETE 0u        // word 0 of a tile: hit lists complete
 #define RGX_REC_OVERFLOWED 1u      //   the region overflowed (record unusable)
 #define RGX_REC_COMPLETE_SUMS 2u   //   hit lists and sample sums complete
@@ -1106,6 +1109,8 @@ struct Recorder {
     bool ovf;       // the region is exhausted
     bool sums;      // every blending iteration so far got a sample-sum slot
     int slot;       // the current iteration's sample-sum slot, or -1
+    uint32_t batch_next = 0; // the next slot of the batch this tile last took from the pool
+    int batch_left = 0;      // slots left in that batch
     __device__ __forceinline__ bool on() const { return reg != nullptr && !ovf; }
     // room for an item and the iteration's trailer?
     __device__ __forceinline__ bool fits(int size)
@@ -1156,9 +1161,16 @@ struct Recorder {
         if (blends && P.sum_next) {
             // every blending iteration asks, also those of a tile that has gone without once: the counter then
             // ends at the launch's whole demand, which is what the next record of this view's shape is sized from
-            uint32_t s = 0;
-            if (threadIdx.x == 0) s = atomicAdd(P.sum_next, 1u);
-            s = (uint32_t)__builtin_amdgcn_readfirstlane((int)s);
+            // (RGX_SUM_SLOT_BATCH slots per request: a request is a round trip to one counter that every tile of the
+            // launch shares, and where iterations are short the tiles spend a good part of their time waiting on it)
+            if (batch_left == 0) {
+                uint32_t s = 0;
+                if (threadIdx.x == 0) s = atomicAdd(P.sum_next, (uint32_t)RGX_SUM_SLOT_BATCH);
+                batch_next = (uint32_t)__builtin_amdgcn_readfirstlane((int)s);
+                batch_left = RGX_SUM_SLOT_BATCH;
+            }
+            const uint32_t s = batch_next++;
+            --batch_left;
             if (sums && s < (uint32_t)P.sum_slots) slot = (int)s;
             else sums = false;
         }

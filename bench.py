@@ -75,6 +75,9 @@ _valu_measured = None
 
 PROBE_KINDS = ("v_fma_f32", "v_add_f32", "v_mov_b32", "v_and_b32", "v_cmp_lt_f32", "v_cndmask_b32", "v_max_f32",
                "v_add_f32_dpp", "v_lshlrev_b32", "v_exp_f32")
+# kinds 10..13 name their registers (160 of them: three wavefronts per SIMD at most): where the operands live matters
+BANK_KINDS = ("v_fma_f32 acc = x * k + acc, fresh x from the other register bank", "v_fma_f32 d = a * b + c, all fresh, banks mixed",
+              "v_fma_f32 d = a * b + c, all fresh, one bank", "v_mul_f32 d = a * b, both fresh")
 
 
 def probe_rate(dev, kind, waves_per_simd, iters=1024, reps=5):
@@ -106,6 +109,7 @@ def valu_measured(dev):
         _valu_measured = dict(value=round(rate, 1), unit="G wave instructions/s", nominal=round(VALU_NOMINAL_GINST, 1),
                               instructions=count, kernel_ms=round(ms, 4), what="independent v_fma_f32, 8 wavefronts per SIMD",
                               fma_at_3_waves_per_simd=round(probe_rate(dev, 0, 3)[0], 1),
+                              fma_accumulate_at_3_waves_per_simd=round(probe_rate(dev, 10, 3)[0], 1),
                               cmp_at_3_waves_per_simd=round(probe_rate(dev, 4, 3)[0], 1),
                               exp_at_3_waves_per_simd=round(probe_rate(dev, 9, 3)[0], 1))
     return _valu_measured
@@ -117,6 +121,8 @@ def valu_cost_table(dev):
     table = {}
     for kind, name in enumerate(PROBE_KINDS):
         table[name] = {str(w): round(1024 * 2.4 / probe_rate(dev, kind, w, reps=3)[0], 2) for w in (1, 2, 3, 4, 8)}
+    for kind, name in enumerate(BANK_KINDS, start=len(PROBE_KINDS)):
+        table[name] = {str(w): round(1024 * 2.4 / probe_rate(dev, kind, w, reps=3)[0], 2) for w in (1, 2, 3)}
     return table
 
 

@@ -1100,6 +1100,25 @@ def test_settings_update_refits_inside_the_render_function(gx):
 
 
 @pytest.mark.gpu
+def test_issue_rate_probe_runs_every_kind(gx):
+    """rgx_probe_valu_rate: every instruction kind (0..9 placed by the compiler, 10..13 with named registers) launches,
+    reports the instruction count of its shape and writes nothing to the sink; kinds out of range are refused."""
+    import ctypes as C
+    from raygaussx_amd import _lib
+    sink = torch.full((4,), 7.0, device=gx.DEV)
+    count = C.c_uint64(0)
+    for kind in range(14):
+        _step(f"issue-rate probe, kind {kind}")
+        _lib.check(_lib.lib().rgx_probe_valu_rate(C.c_int32(1024), C.c_int32(8), C.c_int32(kind), _lib.ptr(sink), C.byref(count),
+                                                  _lib.stream()))
+        torch.cuda.synchronize()
+        assert count.value == 1024 * 8 * 64
+    assert bool((sink == 7.0).all())
+    for kind in (-1, 14):
+        assert _lib.lib().rgx_probe_valu_rate(C.c_int32(1024), C.c_int32(8), C.c_int32(kind), _lib.ptr(sink), C.byref(count),
+                                              _lib.stream()) == -1
+
+
 def test_scratch_of_streams_no_longer_used_is_dropped(gx, c0):
     """The host mirror keeps one set of scratch tensors per stream in use; a loop that keeps making new
     streams must not keep a set for each of them."""

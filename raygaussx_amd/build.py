@@ -5,7 +5,7 @@
 evaluation (fused multiply-adds only where the source says fmaf);
 ``-munsafe-fp-atomics`` selects the hardware fp32 atomic add for the gradient
 scatter; packed-fp32 code generation is disabled; the march kernels' source is compiled without
-machine-code loop-invariant code motion (``SOURCE_FLAGS``).
+machine-code loop-invariant code motion, in two pieces with different scheduling (``UNITS``).
 
 ``python -m raygaussx_amd.build --resources`` also prints what every kernel takes: registers,
 bytes of register spills per lane, LDS.  The march kernels are sized for three wavefronts per SIMD
@@ -23,7 +23,6 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "librgx.so")
-SOURCES = ["rgx_api.hip", "rgx_build.hip", "rgx_pergauss.hip", "rgx_image.hip", "rgx_march.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off", "-fno-fast-math",
          "-munsafe-fp-atomics", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-Wno-unused-command-line-argument"]
@@ -31,7 +30,17 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=o
 # of their slab loops (addresses, constants, selects of wave-uniform values) it pays for with spills inside them:
 # without it the recording forward runs 3-4 % faster (36 -> 20 bytes of spills per lane; the plain forward and
 # the replaying backward lose theirs altogether and run as before).
-SOURCE_FLAGS = {"rgx_march.hip": ["-mllvm", "-disable-machine-licm=1"]}
+NO_LICM = ["-mllvm", "-disable-machine-licm=1"]
+# The march source is compiled twice: once for everything but the backward kernels, without the scheduling pass
+# that runs after register allocation (the forward without a record runs 1-3 % faster on what the first
+# scheduler left), and once for the backward kernels alone, which that pass helps by about 1 %.
+# (source, object name, flags of that compilation)
+UNITS = [("rgx_api.hip", "rgx_api", []), ("rgx_build.hip", "rgx_build", []), ("rgx_pergauss.hip", "rgx_pergauss", []),
+         ("rgx_image.hip", "rgx_image", []),
+         ("rgx_march.hip", "rgx_march", ["-DRGX_MARCH_TU=1", *NO_LICM, "-mllvm", "-enable-post-misched=0"]),
+         ("rgx_march.hip", "rgx_march_bwd", ["-DRGX_MARCH_TU=2", *NO_LICM])]
+# The diagnostic build keeps the march source in one piece (its cycle table is one device variable).
+UNITS_SECTIONS = UNITS[:4] + [("rgx_march.hip", "rgx_march", NO_LICM)]
 
 
 def _resource_table(compiler_output):
@@ -58,19 +67,19 @@ def _resource_table(compiler_output):
     return "\n".join(out)
 
 
-def build(verbose=False, extra=(), lib=LIB, tag="", resources=False):
+def build(verbose=False, extra=(), lib=LIB, tag="", resources=False, units=None):
     """``extra``: more hipcc flags; ``lib`` / ``tag``: write a differently named library and objects;
-    ``resources``: print every kernel's register, spill and LDS use."""
+    ``resources``: print every kernel's register, spill and LDS use; ``units``: the compilations (``UNITS``)."""
     objs = []
     procs = []
     if resources:
         extra = [*extra, "-Rpass-analysis=kernel-resource-usage"]
-    for src in SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", tag + ".o"))
-        cmd = ["hipcc", *FLAGS, *SOURCE_FLAGS.get(src, []), *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    for src, name, flags in (UNITS if units is None else units):
+        obj = os.path.join(CSRC, name + tag + ".o")
+        cmd = ["hipcc", *FLAGS, *flags, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
-        procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
+        procs.append((name, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))
         objs.append(obj)
     failed = False
     for src, p in procs:
@@ -97,7 +106,7 @@ def build_sections(**kw):
     """The diagnostic build with the per-section cycle census of the march kernels compiled in
     (``-DRGX_SECTION_CLOCKS``): ``librgx_sections.so`` beside the product library, which it never replaces.
     ``RGX_LIB_PATH=raygaussx_amd/librgx_sections.so python bench.py --sections`` reads the census."""
-    return build(extra=["-DRGX_SECTION_CLOCKS"], lib=SECTIONS_LIB, tag="_sections", **kw)
+    return build(extra=["-DRGX_SECTION_CLOCKS"], lib=SECTIONS_LIB, tag="_sections", units=UNITS_SECTIONS, **kw)
 
 
 if __name__ == "__main__":

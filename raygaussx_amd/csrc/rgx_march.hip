@@ -47,6 +47,12 @@
 // stack never holds more than QCAP - 96 + 93 < QCAP entries, whatever the scene.
 #define RGX_DFS_MARGIN 160
 #define RGX_LDS_HITS 32    // per-lane list of the stand-alone collect hook
+// This source can be compiled as one translation unit (RGX_MARCH_TU undefined or 0) or as two, so that the
+// backward kernels can be given other compiler flags than the rest: 1 = everything except the three backward
+// kernels, 2 = only those and the function that launches them.
+#ifndef RGX_MARCH_TU
+#define RGX_MARCH_TU 0
+#endif
 // The march kernels are sized (registers and LDS) for three wavefronts per SIMD.
 #ifndef RGX_WAVES_ATTR
 #define RGX_WAVES_ATTR __attribute__((amdgpu_waves_per_eu(3, 3)))
@@ -2226,6 +2232,7 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
     RGX_SEC_FLUSH(cn, REPLAY ? (SUMS ? RGX_SECK_BWD_SUMS : RGX_SECK_BWD_LISTS) : RGX_SECK_BWD_TREE);
 }
 
+#if RGX_MARCH_TU != 2
 // Launch order of the replaying backward.  A tile is one wavefront's work from start to end, so a
 // launch ends with a tail in which ever fewer tiles are still running; the tail is as long as the
 // tiles that start last.  The records say how much work each tile is (words used), so every XCD
@@ -2354,6 +2361,14 @@ __global__ __launch_bounds__(1024) void k_block_order(const MarchParams P, const
     }
 }
 
+#endif // RGX_MARCH_TU != 2
+
+// The three backward kernels are launched through this one function, which lives in the translation unit
+// that holds them.
+enum { RGX_BWD_TREE, RGX_BWD_LISTS, RGX_BWD_SUMS };
+__attribute__((visibility("hidden"))) void rgx_launch_march_bwd(int which, bool stats, bool half, dim3 grid, hipStream_t s,
+                                                                const MarchParams &P);
+#if RGX_MARCH_TU != 1
 // The backward that searches the tree, and the one that replays the forward's record.  (Three
 // waves per SIMD with some spilling measured faster for the replay than two waves without.)
 template <bool STATS>
@@ -2365,6 +2380,26 @@ template <bool STATS, bool HALF = false>
 #define RGX_WAVES_ATTR_SUMS RGX_WAVES_ATTR
 #endif
 __global__ __launch_bounds__(64) RGX_WAVES_ATTR_SUMS void k_march_bwd_replay_sums(const MarchParams P) { march_bwd<true, true, STATS, HALF>(P); }
+
+void rgx_launch_march_bwd(int which, bool stats, bool half, dim3 grid, hipStream_t s, const MarchParams &P)
+{
+    const dim3 wave(64);
+    if (which == RGX_BWD_SUMS) {
+        if (stats && half) hipLaunchKernelGGL((k_march_bwd_replay_sums<true, true>), grid, wave, 0, s, P);
+        else if (stats) hipLaunchKernelGGL((k_march_bwd_replay_sums<true, false>), grid, wave, 0, s, P);
+        else if (half) hipLaunchKernelGGL((k_march_bwd_replay_sums<false, true>), grid, wave, 0, s, P);
+        else hipLaunchKernelGGL((k_march_bwd_replay_sums<false, false>), grid, wave, 0, s, P);
+    } else if (which == RGX_BWD_LISTS) {
+        if (stats) hipLaunchKernelGGL(k_march_bwd_replay<true>, grid, wave, 0, s, P);
+        else hipLaunchKernelGGL(k_march_bwd_replay<false>, grid, wave, 0, s, P);
+    } else {
+        if (stats) hipLaunchKernelGGL(k_march_bwd<true>, grid, wave, 0, s, P);
+        else hipLaunchKernelGGL(k_march_bwd<false>, grid, wave, 0, s, P);
+    }
+}
+#endif // RGX_MARCH_TU != 1
+
+#if RGX_MARCH_TU != 2
 
 // Test hook for the cooperative collect: per pixel a segment [tlo, thi] (thi < tlo = pixel idle);
 // writes each ray's hit count (negated when cut at cap) and the INPUT indices of its hits.
@@ -2760,21 +2795,12 @@ static int march_backward_launch(const void *ws, const RgxCamera *cam, const Rgx
             hipLaunchKernelGGL(k_tile_order, dim3(8), dim3(256), 0, s, P);
             P.use_tile_order = 1;
         }
-        const bool half = P.m.record_format == 1;
-        if (stats) {
-            if (P.sum_pool && half) hipLaunchKernelGGL((k_march_bwd_replay_sums<true, true>), march_grid(P), dim3(64), 0, s, P);
-            else if (P.sum_pool) hipLaunchKernelGGL((k_march_bwd_replay_sums<true, false>), march_grid(P), dim3(64), 0, s, P);
-            hipLaunchKernelGGL(k_march_bwd_replay<true>, march_grid(P), dim3(64), 0, s, P);
-        } else {
-            if (P.sum_pool && half) hipLaunchKernelGGL((k_march_bwd_replay_sums<false, true>), march_grid(P), dim3(64), 0, s, P);
-            else if (P.sum_pool) hipLaunchKernelGGL((k_march_bwd_replay_sums<false, false>), march_grid(P), dim3(64), 0, s, P);
-            hipLaunchKernelGGL(k_march_bwd_replay<false>, march_grid(P), dim3(64), 0, s, P);
-        }
+        if (P.sum_pool) rgx_launch_march_bwd(RGX_BWD_SUMS, stats != nullptr, P.m.record_format == 1, march_grid(P), s, P);
+        rgx_launch_march_bwd(RGX_BWD_LISTS, stats != nullptr, false, march_grid(P), s, P);
         P.only_overflow = 1;
         P.use_tile_order = 0;
     }
-    if (stats) hipLaunchKernelGGL(k_march_bwd<true>, march_grid(P), dim3(64), 0, s, P);
-    else hipLaunchKernelGGL(k_march_bwd<false>, march_grid(P), dim3(64), 0, s, P);
+    rgx_launch_march_bwd(RGX_BWD_TREE, stats != nullptr, false, march_grid(P), s, P);
     rgx_span_end(span, s);
     span = timed ? rgx_span_begin(RGX_T_UNPERMUTE, s) : nullptr;
     hipLaunchKernelGGL(k_unpermute_grads, grid_for(n, 256), dim3(256), 0, s, (const float4 *)P.gbuf, P.order, n, ddens, drgb,
@@ -3025,3 +3051,4 @@ extern "C" int rgx_probe_valu_rate(int32_t waves, int32_t iters, int32_t kind, f
     RGX_LAUNCH_CHECK();
     return RGX_OK;
 }
+#endif // RGX_MARCH_TU != 2

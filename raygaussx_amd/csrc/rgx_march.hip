@@ -1947,6 +1947,42 @@ __device__ __forceinline__ float group_sum(float v)
     return v;
 }
 
+// The 13 sums of a gradient trip over the 8 lanes of a group, in seven registers: r[c] is the group's sum of out[c]
+// in the group's first four lanes and that of out[c + 7] in its last four (r[6] there: undefined).  The step between
+// the two quads of a group writes with a bank mask (a bank = four lanes): the even banks add up component c, the odd
+// banks component c + 7, so that the two steps inside the quads run on seven registers instead of thirteen.
+// (Inline assembly because the compiler has no masked form of the data-parallel add.  The s_nop at either end is the
+// two wait states this chip needs between a vector instruction's write and a data-parallel read of the register:
+// the compiler counts them for its own instructions only.)
+__device__ __forceinline__ void group_sums_split(const float (&out)[RGX_NSUM], float (&r)[7])
+{
+    static_assert(RGX_NSUM == 13, "seven and six");
+    asm volatile("s_nop 1\n\t"
+                 "v_add_f32_dpp %0, %7, %7 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                 "v_add_f32_dpp %1, %8, %8 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                 "v_add_f32_dpp %2, %9, %9 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                 "v_add_f32_dpp %3, %10, %10 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                 "v_add_f32_dpp %4, %11, %11 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                 "v_add_f32_dpp %5, %12, %12 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                 "v_add_f32_dpp %6, %13, %13 row_half_mirror row_mask:0xf bank_mask:0x5\n\t"
+                 "v_add_f32_dpp %0, %14, %14 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                 "v_add_f32_dpp %1, %15, %15 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                 "v_add_f32_dpp %2, %16, %16 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                 "v_add_f32_dpp %3, %17, %17 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                 "v_add_f32_dpp %4, %18, %18 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                 "v_add_f32_dpp %5, %19, %19 row_half_mirror row_mask:0xf bank_mask:0xa\n\t"
+                 "s_nop 1"
+                 : "=&v"(r[0]), "=&v"(r[1]), "=&v"(r[2]), "=&v"(r[3]), "=&v"(r[4]), "=&v"(r[5]), "=&v"(r[6])
+                 : "v"(out[0]), "v"(out[1]), "v"(out[2]), "v"(out[3]), "v"(out[4]), "v"(out[5]), "v"(out[6]), "v"(out[7]),
+                   "v"(out[8]), "v"(out[9]), "v"(out[10]), "v"(out[11]), "v"(out[12]));
+#pragma unroll
+    for (int c = 0; c < 7; ++c) {
+        r[c] += row_take<0xB1>(r[c]); // quad_perm [1,0,3,2]
+        r[c] += row_take<0x4E>(r[c]); // quad_perm [2,3,0,1]
+        asm volatile("" : "+v"(r[c])); // (here, for all lanes: otherwise the last add moves under the condition of the adds to LDS and leaves a move behind)
+    }
+}
+
 // ---------------------------------------------------------------------------
 // Backward: __raygen__rg of cuda_train/backward/gaussians_aabb.cu:209-497.
 //
@@ -1964,8 +2000,9 @@ __device__ __forceinline__ float group_sum(float v)
 // So the inner loop carries three moments (sum y, sum y u, sum y u^2) instead of
 // nineteen running sums; the `power < k^2` mask follows the forward's 32-step recurrence, i.e. it
 // is the mask the forward blended with.  Per Gaussian the moments turn into 13 sums in its whitened
-// frame (RGX_NSUM); those are summed over the 16 rays of a row with DPP adds and carried on by one
-// lane per row; the change of variables to the 14 gradient words comes after all sums.
+// frame (RGX_NSUM); those are summed over the rays of a group of lanes (a row of 16 in the walk by rows, half a
+// row in a replay) with DPP adds and carried on by one lane per group (two in a replay: group_sums_split); the
+// change of variables to the 14 gradient words comes after all sums.
 template <bool REPLAY, bool SUMS, bool STATS, bool HALF = false>
 __device__ __forceinline__ void march_bwd(const MarchParams &P)
 {
@@ -2160,6 +2197,28 @@ __device__ __forceinline__ void march_bwd(const MarchParams &P)
                 }
                 // summed over the group's rays; one lane per group carries the sums on
                 const uint64_t bal = __ballot(hit);
+                if constexpr (REPLAY && GROUP == 8) {
+                    // the group's sums end up in two of its lanes, seven components in the first, six in the fifth
+                    float r[7];
+                    group_sums_split(out, r);
+                    const int first = lane & ~7;
+                    if ((lane & 3) == 0 && live && ((bal >> first) & 0xffull)) {
+                        const bool upper = lane & 4;
+                        if (!upper) {
+                            if constexpr (STATS) {
+                                if (!(atomicOr(&s_pid[e.slot], RGX_SLOT_TOUCHED) & RGX_SLOT_TOUCHED)) cn.grad_atomics += 14;
+                            } else {
+                                atomicOr(&s_pid[e.slot], RGX_SLOT_TOUCHED);
+                            }
+                        }
+                        float *dst = &s_acc[(upper ? 7 * RGX_CCAP : 0) + e.slot];
+#pragma unroll
+                        for (int c = 0; c < 6; ++c) unsafeAtomicAdd(dst + c * RGX_CCAP, r[c]);
+                        if (!upper) unsafeAtomicAdd(dst + 6 * RGX_CCAP, r[6]);
+                    }
+                    RGX_SEC(cn, RGX_SEC_SHADE);
+                    return;
+                }
 #pragma unroll
                 for (int c = 0; c < RGX_NSUM; ++c) out[c] = group_sum<GROUP>(out[c]);
                 if ((lane & (GROUP - 1)) == 0 && live && ((bal >> lane) & ((1ull << GROUP) - 1ull))) {

@@ -6,6 +6,8 @@
 #include "rgx_device.h"
 #include <float.h>
 
+#include <algorithm>
+
 // ---------------------------------------------------------------------------
 // order-preserving float <-> int encoding for atomicMin/atomicMax
 __device__ __forceinline__ int32_t enc_f(float f)
@@ -70,9 +72,10 @@ __global__ __launch_bounds__(256) void k_aabb(const float *__restrict__ pos, con
                                               const float *__restrict__ quat, const float *__restrict__ dens,
                                               int64_t n, float thr, float *__restrict__ boxes, int32_t *mn_enc, int32_t *mx_enc)
 {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    // (a block takes several rounds of 256 Gaussians: every block ends with six atomics on the same six words,
+    // and one per 256 Gaussians made those the kernel's time)
     float b[6] = {INFINITY, INFINITY, INFINITY, -INFINITY, -INFINITY, -INFINITY};
-    if (i < n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
         const float t = dens[i] / thr;
         float d = canon_logf(t * t);
         if (!(d > 0.0f)) d = 0.0f;
@@ -89,10 +92,13 @@ __global__ __launch_bounds__(256) void k_aabb(const float *__restrict__ pos, con
         const float hy = d * sqrtf(((s0 * L2x) * (s0 * L2x) + (s1 * L2y) * (s1 * L2y)) + (s2 * L2z) * (s2 * L2z));
         const float hz = d * sqrtf(((s0 * L3x) * (s0 * L3x) + (s1 * L3y) * (s1 * L3y)) + (s2 * L3z) * (s2 * L3z));
         const float c0 = pos[3 * i], c1 = pos[3 * i + 1], c2 = pos[3 * i + 2];
-        b[0] = c0 - hx; b[1] = c1 - hy; b[2] = c2 - hz;
-        b[3] = c0 + hx; b[4] = c1 + hy; b[5] = c2 + hz;
+        const float e[6] = {c0 - hx, c1 - hy, c2 - hz, c0 + hx, c1 + hy, c2 + hz};
         if (boxes)
-            for (int a = 0; a < 6; ++a) boxes[6 * i + a] = b[a];
+            for (int a = 0; a < 6; ++a) boxes[6 * i + a] = e[a];
+        for (int a = 0; a < 3; ++a) {
+            b[a] = fminf(b[a], e[a]);
+            b[a + 3] = fmaxf(b[a + 3], e[a + 3]);
+        }
     }
     __shared__ float red[4][6];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -193,7 +199,8 @@ __global__ __launch_bounds__(RGX_RS_THREADS) void k_rs_hist(const K *__restrict_
 }
 
 // Exclusive scan of the (digit, tile) counts in two levels: block d scans its digit's row of tile
-// counts in place and leaves the row total; one more block scans the 256 totals into digit bases.
+// counts in place and leaves the row total; every block of the scatter scans the 256 totals into
+// digit bases for itself (a launch of one block for that cost more than 500 blocks doing it again).
 __global__ __launch_bounds__(256) void k_rs_scan_rows(uint32_t *__restrict__ hist, int nblocks, uint32_t *__restrict__ totals)
 {
     __shared__ uint32_t part[256];
@@ -217,31 +224,28 @@ __global__ __launch_bounds__(256) void k_rs_scan_rows(uint32_t *__restrict__ his
     if (threadIdx.x == 0) totals[blockIdx.x] = carry;
 }
 
-__global__ __launch_bounds__(256) void k_rs_scan_totals(uint32_t *__restrict__ totals)
-{
-    __shared__ uint32_t part[256];
-    const uint32_t v = totals[threadIdx.x];
-    part[threadIdx.x] = v;
-    __syncthreads();
-    for (int o = 1; o < 256; o <<= 1) {
-        const uint32_t t = (int)threadIdx.x >= o ? part[threadIdx.x - o] : 0u;
-        __syncthreads();
-        part[threadIdx.x] += t;
-        __syncthreads();
-    }
-    totals[threadIdx.x] = part[threadIdx.x] - v;
-}
-
 template <typename K>
 __global__ __launch_bounds__(RGX_RS_THREADS) void k_rs_scatter(const K *__restrict__ kin, const uint32_t *__restrict__ vin,
                                                                K *__restrict__ kout, uint32_t *__restrict__ vout, int64_t n,
                                                                int shift, const uint32_t *__restrict__ hist, int nblocks,
-                                                               const uint32_t *__restrict__ digit_base)
+                                                               const uint32_t *__restrict__ totals)
 {
+    static_assert(RGX_RS_THREADS == 256, "one thread per digit");
     __shared__ uint32_t cnt[4][256];
+    __shared__ uint32_t wave_total[4];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int w = 0; w < 4; ++w) cnt[w][threadIdx.x] = 0;
+    // digit_base: exclusive scan of the digits' totals, thread d for digit d
+    const uint32_t total = totals[threadIdx.x];
+    uint32_t incl = total;
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t t = __shfl_up(incl, o);
+        if (lane >= o) incl += t;
+    }
+    if (lane == 63) wave_total[wave] = incl;
     __syncthreads();
+    uint32_t digit_base = incl - total;
+    for (int w = 0; w < wave; ++w) digit_base += wave_total[w];
     // wave w owns the contiguous 512 keys [base + 512 w, +512), 64 per round
     const int64_t base = (int64_t)blockIdx.x * RGX_RS_TILE + (int64_t)wave * (64 * RGX_RS_ITEMS);
     K key[RGX_RS_ITEMS];
@@ -259,7 +263,7 @@ __global__ __launch_bounds__(RGX_RS_THREADS) void k_rs_scatter(const K *__restri
     __syncthreads();
     {
         const int d = threadIdx.x;
-        uint32_t run = digit_base[d] + hist[(size_t)d * nblocks + blockIdx.x];
+        uint32_t run = digit_base + hist[(size_t)d * nblocks + blockIdx.x];
         for (int w = 0; w < 4; ++w) {
             const uint32_t c = cnt[w][d];
             cnt[w][d] = run;
@@ -300,7 +304,6 @@ static int radix_sort(K *k0, uint32_t *v0, K *k1, uint32_t *v1, int64_t n, int b
         hipLaunchKernelGGL(k_rs_hist<K>, dim3(nblocks), dim3(RGX_RS_THREADS), 0, s, ki, n, shift, hist, nblocks);
         uint32_t *totals = hist + (size_t)256 * nblocks;
         hipLaunchKernelGGL(k_rs_scan_rows, dim3(256), dim3(256), 0, s, hist, nblocks, totals);
-        hipLaunchKernelGGL(k_rs_scan_totals, dim3(1), dim3(256), 0, s, totals);
         hipLaunchKernelGGL(k_rs_scatter<K>, dim3(nblocks), dim3(RGX_RS_THREADS), 0, s, ki, vi, ko, vo, n, shift, hist, nblocks,
                            totals);
         K *tk = ki; ki = ko; ko = tk;
@@ -314,11 +317,13 @@ static int radix_sort(K *k0, uint32_t *v0, K *k1, uint32_t *v1, int64_t n, int b
 // Leaves, radix tree (Karras 2012), refit, skip links.
 __global__ __launch_bounds__(256) void k_leaves(const float *__restrict__ boxes, const uint32_t *__restrict__ order, int64_t n,
                                                 Node *__restrict__ nodes, int32_t *__restrict__ parent, int32_t *__restrict__ flags,
-                                                const int32_t *gate = nullptr)
+                                                uint32_t *__restrict__ place, const int32_t *gate = nullptr)
 {
     const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (j >= n || gate_closed(gate)) return;
-    const float *b = boxes + 6 * (int64_t)order[j];
+    const int64_t in = order[j];
+    place[in] = (uint32_t)j; // the inverse permutation, for the kernels that go through the Gaussians in input order
+    const float *b = boxes + 6 * in;
     Node nd;
     nd.lo[0] = b[0]; nd.lo[1] = b[1]; nd.lo[2] = b[2];
     nd.hi[0] = b[3]; nd.hi[1] = b[4]; nd.hi[2] = b[5];
@@ -478,6 +483,8 @@ __global__ void k_mark_built(WsHeader *h, const int32_t *gate = nullptr)
 
 // ---------------------------------------------------------------------------
 static inline dim3 grid_for(int64_t n, int block) { return dim3((unsigned)((n + block - 1) / block)); }
+// For the kernels that loop over their input and end with atomics on a few shared words: two blocks per CU.
+static inline dim3 grid_reduce(int64_t n, int block) { return dim3((unsigned)std::min<int64_t>((n + block - 1) / block, 512)); }
 
 extern "C" int rgx_aabb(const float *pos, const float *scale, const float *quat, const float *dens, int64_t n,
                         float sigma_threshold, float *bboxes, float *bb_min, float *bb_max, void *stream)
@@ -489,7 +496,7 @@ extern "C" int rgx_aabb(const float *pos, const float *scale, const float *quat,
     int32_t *mn = (int32_t *)bb_min, *mx = (int32_t *)bb_max;
     if (mn) hipLaunchKernelGGL(k_init_enc, dim3(1), dim3(64), 0, s, mn, mx);
     if (n > 0)
-        hipLaunchKernelGGL(k_aabb, grid_for(n, 256), dim3(256), 0, s, pos, scale, quat, dens, n, sigma_threshold, bboxes, mn, mx);
+        hipLaunchKernelGGL(k_aabb, grid_reduce(n, 256), dim3(256), 0, s, pos, scale, quat, dens, n, sigma_threshold, bboxes, mn, mx);
     if (mn) hipLaunchKernelGGL(k_decode_enc, dim3(1), dim3(64), 0, s, mn, mx);
     RGX_LAUNCH_CHECK();
     return RGX_OK;
@@ -507,10 +514,12 @@ __global__ __launch_bounds__(256) void k_take_boxes(const float *__restrict__ in
                                                     int32_t *mn_enc, int32_t *mx_enc, const int32_t *gate = nullptr)
 {
     if (gate_closed(gate)) return; // the whole grid
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     float b[6] = {INFINITY, INFINITY, INFINITY, -INFINITY, -INFINITY, -INFINITY};
-    if (i < n)
-        for (int a = 0; a < 6; ++a) boxes[6 * i + a] = b[a] = in[6 * i + a];
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        for (int a = 0; a < 6; ++a) {
+            const float v = boxes[6 * i + a] = in[6 * i + a];
+            b[a] = a < 3 ? fminf(b[a], v) : fmaxf(b[a], v);
+        }
     __shared__ float red[4][6];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int a = 0; a < 3; ++a) {
@@ -562,10 +571,10 @@ static int build_impl(const float *pos, const float *scale, const float *quat, c
     hipLaunchKernelGGL(k_init_header, dim3(1), dim3(64), 0, s, hdr, n);
     if (n > 0) {
         if (in_boxes)
-            hipLaunchKernelGGL(k_take_boxes, grid_for(n, 256), dim3(256), 0, s, in_boxes, n, boxes, hdr->bb_min_enc,
+            hipLaunchKernelGGL(k_take_boxes, grid_reduce(n, 256), dim3(256), 0, s, in_boxes, n, boxes, hdr->bb_min_enc,
                                hdr->bb_max_enc);
         else
-            hipLaunchKernelGGL(k_aabb, grid_for(n, 256), dim3(256), 0, s, pos, scale, quat, dens, n, sigma_threshold, boxes,
+            hipLaunchKernelGGL(k_aabb, grid_reduce(n, 256), dim3(256), 0, s, pos, scale, quat, dens, n, sigma_threshold, boxes,
                                hdr->bb_min_enc, hdr->bb_max_enc);
         hipLaunchKernelGGL(k_finish_bbox, dim3(1), dim3(64), 0, s, hdr, (float *)nullptr, (float *)nullptr);
         hipLaunchKernelGGL(k_morton63, grid_for(n, 256), dim3(256), 0, s, boxes, n, hdr, k0, v0);
@@ -573,7 +582,7 @@ static int build_impl(const float *pos, const float *scale, const float *quat, c
         const int r = radix_sort<uint64_t>(k0, v0, k1, v1, n, 64, hist, s);
         if (r < 0) return r;
         // 8 passes: the sorted keys / permutation are back in (k0, v0)
-        hipLaunchKernelGGL(k_leaves, grid_for(n, 256), dim3(256), 0, s, boxes, v0, n, nodes, parent, flags);
+        hipLaunchKernelGGL(k_leaves, grid_for(n, 256), dim3(256), 0, s, boxes, v0, n, nodes, parent, flags, v1); // (the sort's second value buffer is free again)
         if (n > 1) {
             int32_t *other_end = (int32_t *)k1; // the sort's second key buffer is free again
             hipLaunchKernelGGL(k_karras, grid_for(n - 1, 256), dim3(256), 0, s, k0, n, nodes, parent, right, other_end);
@@ -611,9 +620,9 @@ extern "C" int rgx_refit_aabbs(const float *bboxes, int64_t n, void *ws, size_t 
     const int32_t *gate = &hdr->refit_ok;
     hipLaunchKernelGGL(k_refit_begin, dim3(1), dim3(64), 0, s, hdr, n);
     if (n > 0) {
-        hipLaunchKernelGGL(k_take_boxes, grid_for(n, 256), dim3(256), 0, s, bboxes, n, boxes, hdr->bb_min_enc, hdr->bb_max_enc, gate);
+        hipLaunchKernelGGL(k_take_boxes, grid_reduce(n, 256), dim3(256), 0, s, bboxes, n, boxes, hdr->bb_min_enc, hdr->bb_max_enc, gate);
         hipLaunchKernelGGL(k_finish_bbox, dim3(1), dim3(64), 0, s, hdr, (float *)nullptr, (float *)nullptr, gate);
-        hipLaunchKernelGGL(k_leaves, grid_for(n, 256), dim3(256), 0, s, boxes, order, n, nodes, parent, flags, gate);
+        hipLaunchKernelGGL(k_leaves, grid_for(n, 256), dim3(256), 0, s, boxes, order, n, nodes, parent, flags, (uint32_t *)(w + L.vals1), gate);
         if (n > 1) hipLaunchKernelGGL(k_refit, grid_for(n, 256), dim3(256), 0, s, n, nodes, parent, right, other_end, flags, gate);
         hipLaunchKernelGGL(k_skip_links, grid_for(2 * n - 1, 256), dim3(256), 0, s, n, nodes, parent, right, gate);
     }
@@ -676,10 +685,13 @@ extern "C" int rgx_build_order(const void *ws, int64_t n, int32_t *order_out, vo
 // classes/point_cloud.py:1017-1024).
 __global__ __launch_bounds__(256) void k_pos_minmax(const float *__restrict__ pos, int64_t n, int32_t *mn_enc, int32_t *mx_enc)
 {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     float b[6] = {INFINITY, INFINITY, INFINITY, -INFINITY, -INFINITY, -INFINITY};
-    if (i < n)
-        for (int a = 0; a < 3; ++a) b[a] = b[a + 3] = pos[3 * i + a];
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        for (int a = 0; a < 3; ++a) {
+            const float v = pos[3 * i + a];
+            b[a] = fminf(b[a], v);
+            b[a + 3] = fmaxf(b[a + 3], v);
+        }
     __shared__ float red[4][6];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int a = 0; a < 3; ++a) {
@@ -756,7 +768,7 @@ extern "C" int rgx_morton_order(const float *pos, int64_t n, int64_t *codes, int
     uint32_t *k0 = (uint32_t *)(w + L.keys0), *k1 = (uint32_t *)(w + L.keys1);
     uint32_t *v0 = (uint32_t *)(w + L.vals0), *v1 = (uint32_t *)(w + L.vals1);
     hipLaunchKernelGGL(k_init_enc, dim3(1), dim3(64), 0, s, mn, mx);
-    hipLaunchKernelGGL(k_pos_minmax, grid_for(n, 256), dim3(256), 0, s, pos, n, mn, mx);
+    hipLaunchKernelGGL(k_pos_minmax, grid_reduce(n, 256), dim3(256), 0, s, pos, n, mn, mx);
     hipLaunchKernelGGL(k_decode_enc, dim3(1), dim3(64), 0, s, mn, mx);
     hipLaunchKernelGGL(k_morton30, grid_for(n, 256), dim3(256), 0, s, pos, n, (const float *)mn, (const float *)mx, k0, v0, codes);
     RGX_LAUNCH_CHECK();
@@ -960,7 +972,7 @@ extern "C" int rgx_dist2_knn3(const float *pos, int64_t n, float *mean_dist2, vo
     uint32_t *v0 = (uint32_t *)(w + K.m.vals0), *v1 = (uint32_t *)(w + K.m.vals1);
     float4 *pts = (float4 *)(w + K.pts), *boxes = (float4 *)(w + K.boxes), *supers = (float4 *)(w + K.supers);
     hipLaunchKernelGGL(k_init_enc, dim3(1), dim3(64), 0, s, mn, mx);
-    hipLaunchKernelGGL(k_pos_minmax, grid_for(n, 256), dim3(256), 0, s, pos, n, mn, mx);
+    hipLaunchKernelGGL(k_pos_minmax, grid_reduce(n, 256), dim3(256), 0, s, pos, n, mn, mx);
     hipLaunchKernelGGL(k_decode_enc, dim3(1), dim3(64), 0, s, mn, mx);
     hipLaunchKernelGGL(k_morton30, grid_for(n, 256), dim3(256), 0, s, pos, n, (const float *)mn, (const float *)mx, k0, v0,
                        (int64_t *)nullptr);

@@ -124,7 +124,9 @@ struct WsLayout {
 };
 
 #define RGX_RS_THREADS 256
+#ifndef RGX_RS_ITEMS
 #define RGX_RS_ITEMS 8
+#endif
 #define RGX_RS_TILE (RGX_RS_THREADS * RGX_RS_ITEMS)
 
 static inline size_t rgx_align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -139,8 +141,8 @@ static inline WsLayout rgx_ws_layout(int64_t n)
     L.aabb = off;   off = rgx_align_up(off + nn * 6 * sizeof(float), 256);
     L.keys0 = off;  off = rgx_align_up(off + nn * sizeof(uint64_t), 256);
     L.keys1 = off;  off = rgx_align_up(off + nn * sizeof(uint64_t), 256);
-    L.vals0 = off;  off = rgx_align_up(off + nn * sizeof(uint32_t), 256);
-    L.vals1 = off;  off = rgx_align_up(off + nn * sizeof(uint32_t), 256);
+    L.vals0 = off;  off = rgx_align_up(off + nn * sizeof(uint32_t), 256); // after the build: sorted position -> input index
+    L.vals1 = off;  off = rgx_align_up(off + nn * sizeof(uint32_t), 256); // after the build: input index -> sorted position
     L.nodes = off;  off = rgx_align_up(off + (2 * nn) * sizeof(Node), 256);
     L.parent = off; off = rgx_align_up(off + (2 * nn) * sizeof(int32_t), 256);
     L.right = off;  off = rgx_align_up(off + nn * sizeof(int32_t), 256);

@@ -63,7 +63,8 @@ struct MarchParams {
     RgxMarch m;
     const Node *nodes;
     const int32_t *right; // right child of internal node i
-    const uint32_t *order;
+    const uint32_t *order; // sorted position -> input index
+    const uint32_t *place; // input index -> sorted position
     const WsHeader *hdr;
     const Prim *prims;
     int64_t n;
@@ -2506,14 +2507,15 @@ __global__ __launch_bounds__(64) void k_collect_tiles(const MarchParams P, const
 }
 
 // gbuf (Morton order, 16 floats per Gaussian) -> the five gradient tensors in input order
-__global__ __launch_bounds__(256) void k_unpermute_grads(const float4 *__restrict__ gbuf, const uint32_t *__restrict__ order,
+__global__ __launch_bounds__(256) void k_unpermute_grads(const float4 *__restrict__ gbuf, const uint32_t *__restrict__ place,
                                                          int64_t n, float *__restrict__ ddens, float *__restrict__ drgb,
                                                          float *__restrict__ dpos, float *__restrict__ dscale,
                                                          float *__restrict__ dquat)
 {
-    const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (j >= n) return;
-    const int64_t i = order[j];
+    // in input order (place: input index -> sorted position): one 64-byte read wherever it lies, whole lines written
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t j = place[i];
     const float4 a = gbuf[4 * j], b = gbuf[4 * j + 1], c = gbuf[4 * j + 2], d = gbuf[4 * j + 3];
     ddens[i] = a.x;
     drgb[3 * i] = a.y; drgb[3 * i + 1] = a.z; drgb[3 * i + 2] = a.w;
@@ -2607,6 +2609,7 @@ static int fill_params(MarchParams &P, const void *ws, const RgxCamera *cam, con
     P.nodes = (const Node *)(w + L.nodes);
     P.right = (const int32_t *)(w + L.right);
     P.order = (const uint32_t *)(w + L.vals0);
+    P.place = (const uint32_t *)(w + L.vals1);
     P.hdr = (const WsHeader *)(w + L.header);
     P.prims = (const Prim *)prims;
     P.n = n;
@@ -2862,7 +2865,7 @@ static int march_backward_launch(const void *ws, const RgxCamera *cam, const Rgx
     rgx_launch_march_bwd(RGX_BWD_TREE, stats != nullptr, false, march_grid(P), s, P);
     rgx_span_end(span, s);
     span = timed ? rgx_span_begin(RGX_T_UNPERMUTE, s) : nullptr;
-    hipLaunchKernelGGL(k_unpermute_grads, grid_for(n, 256), dim3(256), 0, s, (const float4 *)P.gbuf, P.order, n, ddens, drgb,
+    hipLaunchKernelGGL(k_unpermute_grads, grid_for(n, 256), dim3(256), 0, s, (const float4 *)P.gbuf, P.place, n, ddens, drgb,
                        dpos, dscale, dquat);
     rgx_span_end(span, s);
     RGX_LAUNCH_CHECK();
@@ -2893,6 +2896,7 @@ static int hook_params(MarchParams &P, const void *ws, const float *prims, int64
     P.nodes = (const Node *)(w + L.nodes);
     P.right = (const int32_t *)(w + L.right);
     P.order = (const uint32_t *)(w + L.vals0);
+    P.place = (const uint32_t *)(w + L.vals1);
     P.hdr = (const WsHeader *)(w + L.header);
     P.prims = (const Prim *)prims;
     P.n = n_prims;

@@ -149,12 +149,13 @@ __global__ __launch_bounds__(256) void k_sh_bwd(f3 eye, const float *__restrict_
 // One thread per output record j; reads Gaussian order[j] (or j when order == NULL).
 __global__ __launch_bounds__(256) void k_pack(f3 eye, const float *__restrict__ pos, const float *__restrict__ scale,
                                               const float *__restrict__ quat, const float *__restrict__ dens,
-                                              const float *__restrict__ rgb, const uint32_t *__restrict__ order, int64_t n,
+                                              const float *__restrict__ rgb, const uint32_t *__restrict__ place, int64_t n,
                                               float thr, Prim *__restrict__ prims)
 {
-    const int64_t j = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (j >= n) return;
-    const int64_t i = order ? (int64_t)order[j] : j;
+    // in input order: the five arrays are read in whole cache lines, and a record is one 64-byte write wherever it goes
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t j = place ? (int64_t)place[i] : i;
     const float rho = dens[i];
     const float k = sqrtf(2.0f * canon_logf(rho / thr)); // optix_utils.py:288; NaN below the threshold
     Prim p;
@@ -240,11 +241,11 @@ extern "C" int rgx_pack_prims(const void *ws, const float *eye, const float *pos
     if (!eye || n < 0 || (n > 0 && (!pos || !scale || !quat || !dens || !rgb || !prims)) || ((uintptr_t)prims & 15u))
         return RGX_EINVAL;
     if (n == 0) return RGX_OK;
-    const uint32_t *order = nullptr;
-    if (ws) order = (const uint32_t *)((const char *)ws + rgx_ws_layout(n).vals0);
+    const uint32_t *place = nullptr; // input index -> sorted position
+    if (ws) place = (const uint32_t *)((const char *)ws + rgx_ws_layout(n).vals1);
     void *span = rgx_span_begin(RGX_T_PACK, (hipStream_t)stream);
     hipLaunchKernelGGL(k_pack, grid_for(n, 256), dim3(256), 0, (hipStream_t)stream, f3{eye[0], eye[1], eye[2]}, pos, scale,
-                       quat, dens, rgb, order, n, sigma_threshold, (Prim *)prims);
+                       quat, dens, rgb, place, n, sigma_threshold, (Prim *)prims);
     rgx_span_end(span, (hipStream_t)stream);
     RGX_LAUNCH_CHECK();
     return RGX_OK;

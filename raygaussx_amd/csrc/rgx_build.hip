@@ -431,14 +431,36 @@ __global__ __launch_bounds__(256) void k_refit(int64_t n, Node *nodes, const int
         for (int c = 0; c < 3; ++c) {
             lo[c] = fminf(lo[c], s_box[1 - side][c][slot]);
             hi[c] = fmaxf(hi[c], s_box[1 - side][3 + c][slot]);
-            st_agent(&nodes[node].lo[c], lo[c]);
-            st_agent(&nodes[node].hi[c], hi[c]);
         }
         child = node;
         node = parent[node];
+        // This box is read again inside this kernel only if the parent is met through memory (then by whichever
+        // thread arrives there second, maybe on another XCD): only then does it have to go out as agent-scope
+        // stores.  Everything below such a subtree root is next read by other kernels: plain stores.
+        bool inside = false;
+        if (node >= 0) {
+            const int32_t o = other_end[node];
+            inside = (node < o ? node : o) >= b0 && (node < o ? o : node) <= b1;
+        }
+        if (inside) {
+            for (int c = 0; c < 3; ++c) {
+                nodes[child].lo[c] = lo[c];
+                nodes[child].hi[c] = hi[c];
+            }
+        } else {
+            for (int c = 0; c < 3; ++c) {
+                st_agent(&nodes[child].lo[c], lo[c]);
+                st_agent(&nodes[child].hi[c], hi[c]);
+            }
+            break;
+        }
     }
-    // the rest of the way: through memory
+    // the rest of the way: through memory.  The thread carries its child's box in registers and reads only the
+    // sibling's; the indices it will need after the counter (children, next parent) are asked for before the wait,
+    // so that each level is three trips to memory one after the other (stores acknowledged, counter, sibling's box)
+    // and not five.
     while (node >= 0) {
+        const int32_t left = nodes[node].left, rgt = right[node], up = parent[node];
 #if defined(__gfx942__) || defined(__gfx950__)
         // (the immediate below is the gfx9 encoding of vmcnt(0) with the other counters left alone, and the
         // argument that the wait suffices rests on how these chips complete agent-scope atomic stores)
@@ -451,13 +473,15 @@ __global__ __launch_bounds__(256) void k_refit(int64_t n, Node *nodes, const int
         if (atomicAdd(&flags[node], 1) == 0) return;
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 #endif
-        const Node *a = &nodes[nodes[node].left];
-        const Node *b = &nodes[right[node]];
+        const Node *sibling = &nodes[left == child ? rgt : left];
         for (int c = 0; c < 3; ++c) {
-            st_agent(&nodes[node].lo[c], fminf(ld_agent(&a->lo[c]), ld_agent(&b->lo[c])));
-            st_agent(&nodes[node].hi[c], fmaxf(ld_agent(&a->hi[c]), ld_agent(&b->hi[c])));
+            lo[c] = fminf(lo[c], ld_agent(&sibling->lo[c]));
+            hi[c] = fmaxf(hi[c], ld_agent(&sibling->hi[c]));
+            st_agent(&nodes[node].lo[c], lo[c]);
+            st_agent(&nodes[node].hi[c], hi[c]);
         }
-        node = parent[node];
+        child = node;
+        node = up;
     }
 }
 

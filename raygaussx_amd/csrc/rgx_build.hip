@@ -261,13 +261,31 @@ __global__ __launch_bounds__(RGX_RS_THREADS) void k_rs_scatter(const K *__restri
         }
     }
     __syncthreads();
+    // The tile's keys are put in digit order in LDS first and leave from there: keys of one digit are neighbours
+    // in the tile's order as they are in the output, so thread after thread writes consecutive words instead of
+    // 64 lanes writing to as many streams.  local: where a (wave, digit) run starts in the tile's order;
+    // delta[d]: output position minus position in the tile's order, for digit d.
+    __shared__ uint32_t delta[256];
+    __shared__ K lkey[RGX_RS_TILE];
+    __shared__ uint32_t lval[RGX_RS_TILE];
     {
         const int d = threadIdx.x;
-        uint32_t run = digit_base + hist[(size_t)d * nblocks + blockIdx.x];
+        uint32_t c[4], tile_count = 0;
+        for (int w = 0; w < 4; ++w) tile_count += c[w] = cnt[w][d];
+        uint32_t upto = tile_count; // inclusive scan of the tile's digit counts
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t t = __shfl_up(upto, o);
+            if (lane >= o) upto += t;
+        }
+        __syncthreads(); // (wave_total's first use is over)
+        if (lane == 63) wave_total[wave] = upto;
+        __syncthreads();
+        uint32_t local = upto - tile_count;
+        for (int w = 0; w < wave; ++w) local += wave_total[w];
+        delta[d] = digit_base + hist[(size_t)d * nblocks + blockIdx.x] - local;
         for (int w = 0; w < 4; ++w) {
-            const uint32_t c = cnt[w][d];
-            cnt[w][d] = run;
-            run += c;
+            cnt[w][d] = local;
+            local += c[w];
         }
     }
     __syncthreads();
@@ -285,12 +303,21 @@ __global__ __launch_bounds__(RGX_RS_THREADS) void k_rs_scatter(const K *__restri
         if (valid) {
             const uint32_t rank = __popcll(same & ((1ull << lane) - 1ull));
             const uint32_t off = cur[d];
-            kout[off + rank] = key[r];
-            vout[off + rank] = val[r];
+            lkey[off + rank] = key[r];
+            lval[off + rank] = val[r];
         }
         __builtin_amdgcn_wave_barrier();
         if (valid && (same & ((1ull << lane) - 1ull)) == 0) cur[d] += __popcll(same);
         __builtin_amdgcn_wave_barrier();
+    }
+    __syncthreads();
+    const int64_t tile_base = (int64_t)blockIdx.x * RGX_RS_TILE;
+    const int tile_n = (int)(n - tile_base < RGX_RS_TILE ? n - tile_base : RGX_RS_TILE);
+    for (int p = threadIdx.x; p < tile_n; p += RGX_RS_THREADS) {
+        const K k = lkey[p];
+        const uint32_t out = (uint32_t)p + delta[(uint32_t)(k >> shift) & 255u];
+        kout[out] = k;
+        vout[out] = lval[p];
     }
 }
 

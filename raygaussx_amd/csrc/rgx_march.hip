@@ -2357,34 +2357,45 @@ __global__ __launch_bounds__(256) void k_zero_u32(uint32_t *p, int n)
     if (i < n) p[i] = 0u;
 }
 
-__global__ __launch_bounds__(256) void k_block_cost(const MarchParams P, uint32_t *__restrict__ cost)
+// (A workgroup takes a run of consecutive Gaussians and counts in LDS first: the adds of all workgroups to the few
+// blocks in the middle of the image, one after the other in memory, were three quarters of this kernel's time.)
+#define RGX_COST_BINS 2048
+__global__ __launch_bounds__(256) void k_block_cost(const MarchParams P, uint32_t *__restrict__ cost, int nb, int per_group)
 {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    __shared__ uint32_t s_cost[RGX_COST_BINS];
+    for (int b = threadIdx.x; b < nb; b += 256) s_cost[b] = 0u;
+    __syncthreads();
     const TileGrid g = tile_grid(P.tiles_x, P.tiles_y);
-    int block = -1;
-    if (i < P.n) {
-        const float4 pos4 = P.prims[i].pos4;   // eye - centre
-        const float k = P.prims[i].inv_inter4.w;
-        const f3 c = mk3(-pos4.x, -pos4.y, -pos4.z);
-        const float z = dot3(c, mk3(P.cam.w[0], P.cam.w[1], P.cam.w[2]));
-        if (k == k && z > 1e-6f) { // visible at all, and in front of the camera
-            const float x = dot3(c, mk3(P.cam.u[0], P.cam.u[1], P.cam.u[2])) / z, y = dot3(c, mk3(P.cam.v[0], P.cam.v[1], P.cam.v[2])) / z;
-            const float fx = (x / (2.0f * P.cam.tan_half_fov_x) + P.cam.principal_x) * (float)P.cam.width;
-            const float fy = (y / (2.0f * P.cam.tan_half_fov_y) + P.cam.principal_y) * (float)P.cam.height;
-            if (fx >= 0.f && fx < (float)P.cam.width && fy >= 0.f && fy < (float)P.cam.height)
-                block = (((int)fy >> 3) / g.bh) * g.blocks_x + ((int)fx >> 3) / g.bw;
+    const int64_t first = (int64_t)blockIdx.x * per_group;
+    for (int64_t i = first + threadIdx.x; i < first + per_group; i += 256) { // (per_group is a multiple of 256: whole waves)
+        int block = -1;
+        if (i < P.n) {
+            const float4 pos4 = P.prims[i].pos4;   // eye - centre
+            const float k = P.prims[i].inv_inter4.w;
+            const f3 c = mk3(-pos4.x, -pos4.y, -pos4.z);
+            const float z = dot3(c, mk3(P.cam.w[0], P.cam.w[1], P.cam.w[2]));
+            if (k == k && z > 1e-6f) { // visible at all, and in front of the camera
+                const float x = dot3(c, mk3(P.cam.u[0], P.cam.u[1], P.cam.u[2])) / z, y = dot3(c, mk3(P.cam.v[0], P.cam.v[1], P.cam.v[2])) / z;
+                const float fx = (x / (2.0f * P.cam.tan_half_fov_x) + P.cam.principal_x) * (float)P.cam.width;
+                const float fy = (y / (2.0f * P.cam.tan_half_fov_y) + P.cam.principal_y) * (float)P.cam.height;
+                if (fx >= 0.f && fx < (float)P.cam.width && fy >= 0.f && fy < (float)P.cam.height)
+                    block = (((int)fy >> 3) / g.bh) * g.blocks_x + ((int)fx >> 3) / g.bw;
+            }
+        }
+        // Gaussians are in Morton order, so a wavefront's mostly fall into a few blocks: one add per block
+        uint64_t todo = __ballot(block >= 0);
+        const int lane = threadIdx.x & 63;
+        while (todo) {
+            const int lead = __builtin_ctzll(todo);
+            const int b = __builtin_amdgcn_readlane(block, lead);
+            const uint64_t same = __ballot(block == b);
+            if (lane == lead) atomicAdd(&s_cost[b], (uint32_t)__popcll(same));
+            todo &= ~same;
         }
     }
-    // Gaussians are in Morton order, so a wavefront's mostly fall into a few blocks: one add per block
-    uint64_t todo = __ballot(block >= 0);
-    const int lane = threadIdx.x & 63;
-    while (todo) {
-        const int lead = __builtin_ctzll(todo);
-        const int b = __builtin_amdgcn_readlane(block, lead);
-        const uint64_t same = __ballot(block == b);
-        if (lane == lead) atomicAdd(&cost[b], (uint32_t)__popcll(same));
-        todo &= ~same;
-    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < nb; b += 256)
+        if (s_cost[b]) atomicAdd(&cost[b], s_cost[b]);
 }
 
 __global__ __launch_bounds__(1024) void k_block_order(const MarchParams P, const uint32_t *__restrict__ cost, uint32_t *__restrict__ order)
@@ -2684,7 +2695,9 @@ static void order_blocks(MarchParams &P, hipStream_t s)
     const int nb = g.blocks_x * ((P.tiles_y + g.bh - 1) / g.bh);
     uint32_t *order = P.tile_order, *cost = P.tile_order + 8 * g.per_xcd;
     hipLaunchKernelGGL(k_zero_u32, dim3((unsigned)((nb + 255) / 256)), dim3(256), 0, s, cost, nb);
-    hipLaunchKernelGGL(k_block_cost, dim3((unsigned)((P.n + 255) / 256)), dim3(256), 0, s, P, cost);
+    if (nb > RGX_COST_BINS) return; // (a very long, thin image: as launched)
+    const int per_group = (int)((((P.n + 511) / 512) + 255) / 256 * 256); // 512 workgroups at most, whole waves
+    hipLaunchKernelGGL(k_block_cost, dim3((unsigned)((P.n + per_group - 1) / per_group)), dim3(256), 0, s, P, cost, nb, per_group);
     hipLaunchKernelGGL(k_block_order, dim3(1), dim3(1024), 0, s, P, cost, order);
     P.use_tile_order = 2;
 }

@@ -36,18 +36,17 @@ __device__ __forceinline__ void sh_basis(float x, float y, float z, float *b)
     }
 }
 
+// The colour of one Gaussian (sh_utils.cu:122-216).  coeff: its coefficients, Ks per channel.
 template <int DEG>
-__global__ __launch_bounds__(256) void k_sh_fwd(f3 eye, const float *__restrict__ pos, const float *__restrict__ sh,
-                                                const float *__restrict__ sg, const float *__restrict__ sharp,
-                                                const float *__restrict__ axis, int G, int Gs, int Ks, int64_t n,
-                                                float *__restrict__ rgb)
+__device__ __forceinline__ void sh_fwd_one(f3 eye, const float *__restrict__ pos, const float *__restrict__ coeff,
+                                           const float *__restrict__ sg, const float *__restrict__ sharp,
+                                           const float *__restrict__ axis, int G, int Gs, int Ks, int64_t i,
+                                           float *__restrict__ rgb)
 {
     // Gs, Ks: lobes / coefficients STORED per Gaussian and channel (>= G, >= K): the viewer keeps
     // room for the largest model and evaluates the first G lobes and K coefficients (gui_sh,
     // sh_utils.cu:25-119); everywhere else they equal G and K.
     constexpr int K = (DEG + 1) * (DEG + 1);
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) return;
     const f3 v = mk3(pos[3 * i] - eye.x, pos[3 * i + 1] - eye.y, pos[3 * i + 2] - eye.z);
     const float len = sqrtf(dot3(v, v));
     const f3 d = mk3(v.x / len, v.y / len, v.z / len);
@@ -60,7 +59,7 @@ __global__ __launch_bounds__(256) void k_sh_fwd(f3 eye, const float *__restrict_
     float b[K];
     sh_basis<DEG>(d.x, d.y, d.z, b);
     for (int c = 0; c < 3; ++c) {
-        const float *s = sh + (i * 3 + c) * Ks;
+        const float *s = coeff + c * Ks;
         float r = res[c];
 #pragma unroll
         for (int j = 0; j < K; ++j) r += b[j] * s[j];
@@ -69,18 +68,49 @@ __global__ __launch_bounds__(256) void k_sh_fwd(f3 eye, const float *__restrict_
 }
 
 template <int DEG>
-__global__ __launch_bounds__(256) void k_sh_bwd(f3 eye, const float *__restrict__ pos, const float *__restrict__ sh,
+__global__ __launch_bounds__(256) void k_sh_fwd(f3 eye, const float *__restrict__ pos, const float *__restrict__ sh,
                                                 const float *__restrict__ sg, const float *__restrict__ sharp,
-                                                const float *__restrict__ axis, int G, int64_t n,
-                                                const float *__restrict__ drgb, float *__restrict__ dsh,
-                                                float *__restrict__ dpos, float *__restrict__ dsg,
-                                                float *__restrict__ dsharp, float *__restrict__ daxis)
+                                                const float *__restrict__ axis, int G, int Gs, int Ks, int64_t n,
+                                                float *__restrict__ rgb)
 {
-    constexpr int K = (DEG + 1) * (DEG + 1);
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
+    sh_fwd_one<DEG>(eye, pos, sh + i * 3 * Ks, sg, sharp, axis, G, Gs, Ks, i, rgb);
+}
+
+// Degree 3 with 16 coefficients stored per channel: the 192-byte rows of a workgroup's 256 Gaussians staged in LDS
+// (see k_sh_bwd3_rows).
+__global__ __launch_bounds__(256) void k_sh_fwd3_rows(f3 eye, const float *__restrict__ pos, const float *__restrict__ sh,
+                                                      const float *__restrict__ sg, const float *__restrict__ sharp,
+                                                      const float *__restrict__ axis, int G, int Gs, int64_t n,
+                                                      float *__restrict__ rgb)
+{
+    constexpr int ROW4 = 12, STRIDE4 = 13;
+    __shared__ float4 s_rows[256 * STRIDE4];
+    const int64_t i0 = (int64_t)blockIdx.x * 256;
+    const int rows = (int)(n - i0 < 256 ? n - i0 : 256);
+    const float4 *src = (const float4 *)sh + i0 * ROW4;
+    for (int g = threadIdx.x; g < rows * ROW4; g += 256) {
+        const int r = g / ROW4;
+        s_rows[r * STRIDE4 + (g - r * ROW4)] = src[g];
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < rows)
+        sh_fwd_one<3>(eye, pos, (const float *)&s_rows[threadIdx.x * STRIDE4], sg, sharp, axis, G, Gs, 16, i0 + threadIdx.x, rgb);
+}
+
+// The gradient of one Gaussian (sh_utils.cu:218-412).  coeff: its 3 K coefficients; o_sh: where their gradient goes
+// (may be the same memory: every coefficient is read before the first gradient is written).
+template <int DEG>
+__device__ __forceinline__ void sh_bwd_one(f3 eye, const float *__restrict__ pos, const float *coeff,
+                                           const float *__restrict__ sg, const float *__restrict__ sharp,
+                                           const float *__restrict__ axis, int G, int64_t i,
+                                           const float *__restrict__ drgb, float *o_sh,
+                                           float *__restrict__ dpos, float *__restrict__ dsg,
+                                           float *__restrict__ dsharp, float *__restrict__ daxis)
+{
+    constexpr int K = (DEG + 1) * (DEG + 1);
     const float gr[3] = {drgb[3 * i], drgb[3 * i + 1], drgb[3 * i + 2]};
-    float *o_sh = dsh + i * 3 * K;
     if (gr[0] == 0.f && gr[1] == 0.f && gr[2] == 0.f) { // sh_utils.cu:226 (outputs stay zero)
         for (int j = 0; j < 3 * K; ++j) o_sh[j] = 0.f;
         dpos[3 * i] = dpos[3 * i + 1] = dpos[3 * i + 2] = 0.f;
@@ -95,14 +125,11 @@ __global__ __launch_bounds__(256) void k_sh_bwd(f3 eye, const float *__restrict_
     const float x = v.x / len, y = v.y / len, z = v.z / len;
     float b[K];
     sh_basis<DEG>(x, y, z, b);
-    for (int c = 0; c < 3; ++c)
-#pragma unroll
-        for (int j = 0; j < K; ++j) o_sh[c * K + j] = b[j] * gr[c];
     float dx[3] = {0, 0, 0}, dy[3] = {0, 0, 0}, dz[3] = {0, 0, 0};
     if constexpr (DEG > 0) {
         const float xx = x * x, yy = y * y, zz = z * z, xy = x * y, yz = y * z, xz = x * z;
         for (int c = 0; c < 3; ++c) {
-            const float *s = sh + (i * 3 + c) * K;
+            const float *s = coeff + c * K;
             dx[c] = -SH_C1 * s[3]; dy[c] = -SH_C1 * s[1]; dz[c] = SH_C1 * s[2];
             if constexpr (DEG > 1) {
                 dx[c] += SH_C2[0] * y * s[4] + SH_C2[2] * 2.0f * -x * s[6] + SH_C2[3] * z * s[7] + SH_C2[4] * 2.0f * x * s[8];
@@ -123,6 +150,10 @@ __global__ __launch_bounds__(256) void k_sh_bwd(f3 eye, const float *__restrict_
             }
         }
     }
+    // (the coefficients have all been read: `o_sh` may be the memory `coeff` points to)
+    for (int c = 0; c < 3; ++c)
+#pragma unroll
+        for (int j = 0; j < K; ++j) o_sh[c * K + j] = b[j] * gr[c];
     f3 ddir = mk3((gr[0] * dx[0] + gr[1] * dx[1]) + gr[2] * dx[2], (gr[0] * dy[0] + gr[1] * dy[1]) + gr[2] * dy[2],
                   (gr[0] * dz[0] + gr[1] * dz[1]) + gr[2] * dz[2]);
     for (int l = 0; l < G; ++l) { // sh_utils.cu:385-405
@@ -144,6 +175,51 @@ __global__ __launch_bounds__(256) void k_sh_bwd(f3 eye, const float *__restrict_
     dpos[3 * i + 0] = ((sum2 - v.x * v.x) * ddir.x - v.y * v.x * ddir.y - v.z * v.x * ddir.z) * inv32;
     dpos[3 * i + 1] = (-v.x * v.y * ddir.x + (sum2 - v.y * v.y) * ddir.y - v.z * v.y * ddir.z) * inv32;
     dpos[3 * i + 2] = (-v.x * v.z * ddir.x - v.y * v.z * ddir.y + (sum2 - v.z * v.z) * ddir.z) * inv32;
+}
+
+template <int DEG>
+__global__ __launch_bounds__(256) void k_sh_bwd(f3 eye, const float *__restrict__ pos, const float *__restrict__ sh,
+                                                const float *__restrict__ sg, const float *__restrict__ sharp,
+                                                const float *__restrict__ axis, int G, int64_t n,
+                                                const float *__restrict__ drgb, float *__restrict__ dsh,
+                                                float *__restrict__ dpos, float *__restrict__ dsg,
+                                                float *__restrict__ dsharp, float *__restrict__ daxis)
+{
+    constexpr int K = (DEG + 1) * (DEG + 1);
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    sh_bwd_one<DEG>(eye, pos, sh + i * 3 * K, sg, sharp, axis, G, i, drgb, dsh + i * 3 * K, dpos, dsg, dsharp, daxis);
+}
+
+// Degree 3 (48 coefficients, 192 bytes per Gaussian) with the rows of a workgroup's 256 Gaussians staged in LDS: the
+// workgroup reads and writes its 48 KiB of coefficients and gradients as consecutive 16-byte pieces, lane after lane,
+// instead of 64 lanes each working through a 192-byte row of its own (the same bytes, a quarter of the requests).
+// Rows are 13 float4 apart in LDS, so that the 8 lanes an LDS access serves together fall into different banks.
+__global__ __launch_bounds__(256) void k_sh_bwd3_rows(f3 eye, const float *__restrict__ pos, const float *__restrict__ sh,
+                                                      const float *__restrict__ sg, const float *__restrict__ sharp,
+                                                      const float *__restrict__ axis, int G, int64_t n,
+                                                      const float *__restrict__ drgb, float *__restrict__ dsh,
+                                                      float *__restrict__ dpos, float *__restrict__ dsg,
+                                                      float *__restrict__ dsharp, float *__restrict__ daxis)
+{
+    constexpr int ROW4 = 12, STRIDE4 = 13;
+    __shared__ float4 s_rows[256 * STRIDE4];
+    const int64_t i0 = (int64_t)blockIdx.x * 256;
+    const int rows = (int)(n - i0 < 256 ? n - i0 : 256);
+    const float4 *src = (const float4 *)sh + i0 * ROW4;
+    for (int g = threadIdx.x; g < rows * ROW4; g += 256) {
+        const int r = g / ROW4;
+        s_rows[r * STRIDE4 + (g - r * ROW4)] = src[g];
+    }
+    __syncthreads();
+    float *row = (float *)&s_rows[threadIdx.x * STRIDE4];
+    if ((int)threadIdx.x < rows) sh_bwd_one<3>(eye, pos, row, sg, sharp, axis, G, i0 + threadIdx.x, drgb, row, dpos, dsg, dsharp, daxis);
+    __syncthreads();
+    float4 *dst = (float4 *)dsh + i0 * ROW4;
+    for (int g = threadIdx.x; g < rows * ROW4; g += 256) {
+        const int r = g / ROW4;
+        dst[g] = s_rows[r * STRIDE4 + (g - r * ROW4)];
+    }
 }
 
 // One thread per output record j; reads Gaussian order[j] (or j when order == NULL).
@@ -185,7 +261,12 @@ static int sh_forward_launch(const float *eye, const float *pos, const float *sh
     case 0: hipLaunchKernelGGL(k_sh_fwd<0>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, gs, ks, n, rgb); break;
     case 1: hipLaunchKernelGGL(k_sh_fwd<1>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, gs, ks, n, rgb); break;
     case 2: hipLaunchKernelGGL(k_sh_fwd<2>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, gs, ks, n, rgb); break;
-    default: hipLaunchKernelGGL(k_sh_fwd<3>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, gs, ks, n, rgb); break;
+    default:
+        if (ks == 16 && ((uintptr_t)sh & 15u) == 0)
+            hipLaunchKernelGGL(k_sh_fwd3_rows, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, gs, n, rgb);
+        else
+            hipLaunchKernelGGL(k_sh_fwd<3>, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, gs, ks, n, rgb);
+        break;
     }
     rgx_span_end(span, s);
     RGX_LAUNCH_CHECK();
@@ -225,7 +306,12 @@ extern "C" int rgx_sh_backward(const float *eye, const float *pos, const float *
     case 0: RGX_SHB(0); break;
     case 1: RGX_SHB(1); break;
     case 2: RGX_SHB(2); break;
-    default: RGX_SHB(3); break;
+    default:
+        if ((((uintptr_t)sh | (uintptr_t)dsh) & 15u) == 0)
+            hipLaunchKernelGGL(k_sh_bwd3_rows, grid, block, 0, s, e, pos, sh, sg, sharp, axis, g, n, drgb, dsh, dpos, dsg, dsharp, daxis);
+        else
+            RGX_SHB(3);
+        break;
     }
 #undef RGX_SHB
     rgx_span_end(span, s);
